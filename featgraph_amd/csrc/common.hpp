@@ -1,0 +1,87 @@
+// Shared declarations of libfeatgraph_hip.so: error reporting, tuning store,
+// kernel argument blocks and the launchers that api.hip calls.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/featgraph_hip.h"
+
+namespace fg {
+
+// Records a message for fg_last_error() and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define FG_HIP_TRY(expr)                                                                      \
+  do {                                                                                        \
+    hipError_t fg_err_ = (expr);                                                              \
+    if (fg_err_ != hipSuccess) return ::fg::fail(FG_EHIP, "%s: %s", #expr, hipGetErrorString(fg_err_)); \
+  } while (0)
+
+// Launch-shape overrides (0 = library default).
+struct Config {
+  int spmm_vec = 0, spmm_lpr = 0, spmm_unroll = 0, spmm_scalar_path = -1, spmm_sorted = -1;
+  int sddmm_group = 0, sddmm_batches = 0;
+};
+Config &config();
+
+constexpr int kWaveSize = 64;
+constexpr int kWavesPerBlock = 4;
+constexpr int kBlockThreads = kWaveSize * kWavesPerBlock;
+
+// One launch of the row-slot SpMM kernel.  A "slot" is a group of `lpr` lanes
+// that owns one (row, feature tile) pair.
+struct SpmmArgs {
+  const int32_t *indptr;
+  const int32_t *indices;
+  const float *w;  // [nnz, H] edge weights (H == 1: the CSR values)
+  const float *feat;
+  float *out;
+  const int32_t *row_order;  // rows by descending degree, or null for natural order
+  int32_t n_rows;
+  int32_t F;  // floats per feature row (= H * D)
+  int32_t H;
+  int32_t D;
+  int32_t n_tiles;
+  int64_t n_slots;  // n_tiles * n_rows
+};
+
+struct SpmmShape {
+  int vec, lpr, unroll, scalar_path;
+  int tile_width() const { return vec * lpr; }
+};
+
+SpmmShape spmm_choose_shape(const SpmmArgs &a, int feat_tiles);
+int spmm_launch(const SpmmArgs &a, const SpmmShape &s, hipStream_t stream);
+
+// One launch of the edge-parallel SDDMM kernel over n_ve = nnz * H dot
+// products of length D ("virtual edges": edge e, head h -> e * H + h).
+struct SddmmArgs {
+  const int32_t *row;
+  const int32_t *col;
+  const float *src;
+  const float *dst;
+  float *out;
+  int64_t n_ve;
+  int32_t H;
+  int32_t D;
+  int32_t stride;  // floats per vertex row (= H * D)
+  int32_t batches;  // 64-dot batches per wave
+};
+
+struct SddmmShape {
+  int vec, group, batches;
+};
+
+SddmmShape sddmm_choose_shape(const SddmmArgs &a);
+int sddmm_launch(const SddmmArgs &a, const SddmmShape &s, hipStream_t stream);
+
+inline bool aligned_to(const void *p, uintptr_t bytes) { return (reinterpret_cast<uintptr_t>(p) & (bytes - 1)) == 0; }
+
+inline int pow2_ceil(int x) {
+  int p = 1;
+  while (p < x) p <<= 1;
+  return p;
+}
+
+}  // namespace fg

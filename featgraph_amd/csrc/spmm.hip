@@ -1,0 +1,297 @@
+// CSR SpMM for gfx950: Out[r,:] = sum_e w[e] * Feat[indices[e],:].
+//
+// Work decomposition.  The feature dimension is cut into tiles of
+// TW = VEC * LPR floats.  A "slot" of LPR adjacent lanes owns one (row, tile)
+// pair; every lane of the slot owns VEC adjacent output floats and walks the
+// row's nonzeros from first to last, so each output element is the float32
+// sum of its terms in CSR order starting from +0, with one rounded multiply
+// and one rounded add per term (this file is compiled with -ffp-contract=off).
+// That is the order and rounding of the reference's loop nest
+// (op/vanilla_spmm.py:46-56 with the reorder at :73), so results do not depend
+// on VEC, LPR, the unroll depth or the row schedule.
+//
+// Memory behaviour.  A gather of one neighbour row is LPR lanes * VEC floats
+// of consecutive addresses (TW*4 bytes, 256 B..1 KB), i.e. whole cache lines.
+// Column ids and values of a row are fetched LPR at a time with one coalesced
+// load per slot and handed to the slot's lanes through cross-lane reads, so the
+// index stream is read once per tile.  U independent gathers are issued before
+// the U dependent adds, which is what hides the L2 / Infinity-Cache latency.
+// Slots are numbered tile-major, so at any time the running waves gather from
+// one TW-wide column band of the feature matrix (n_cols * TW * 4 bytes), which
+// is the working set the Infinity Cache has to hold.
+//
+// Row schedule.  Rows are visited by descending degree (the plan's row list):
+// the waves that start first take the hub rows, and the rows that share a wave
+// (64 / LPR of them) have nearly equal lengths, so divergence inside a wave is
+// small.
+#include "common.hpp"
+
+namespace fg {
+namespace {
+
+template <int VEC>
+struct VecOf;
+template <>
+struct VecOf<1> {
+  using type = float;
+};
+template <>
+struct VecOf<2> {
+  using type = float2;
+};
+template <>
+struct VecOf<4> {
+  using type = float4;
+};
+
+template <int VEC>
+__device__ __forceinline__ typename VecOf<VEC>::type vzero();
+template <>
+__device__ __forceinline__ float vzero<1>() {
+  return 0.0f;
+}
+template <>
+__device__ __forceinline__ float2 vzero<2>() {
+  return make_float2(0.0f, 0.0f);
+}
+template <>
+__device__ __forceinline__ float4 vzero<4>() {
+  return make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+}
+
+// acc = acc + v * x, element by element, unfused.
+__device__ __forceinline__ void axpy(float &acc, float v, float x) { acc = acc + v * x; }
+__device__ __forceinline__ void axpy(float2 &acc, float v, float2 x) {
+  acc.x = acc.x + v * x.x;
+  acc.y = acc.y + v * x.y;
+}
+__device__ __forceinline__ void axpy(float4 &acc, float v, float4 x) {
+  acc.x = acc.x + v * x.x;
+  acc.y = acc.y + v * x.y;
+  acc.z = acc.z + v * x.z;
+  acc.w = acc.w + v * x.w;
+}
+
+// Value held by lane `src` of the calling lane's LPR-wide slot.
+template <int LPR>
+__device__ __forceinline__ int slot_read(int v, int src, int lane) {
+  const int from = (lane & ~(LPR - 1)) | src;
+  return __builtin_amdgcn_ds_bpermute(from << 2, v);
+}
+
+// General kernel: 64 / LPR slots per wave, per-lane gather addresses.
+template <int VEC, int LPR, int U, bool MH>
+__global__ __launch_bounds__(kBlockThreads) void spmm_slot_kernel(const SpmmArgs a) {
+  using V = typename VecOf<VEC>::type;
+  constexpr int RPW = kWaveSize / LPR;
+  constexpr int TW = VEC * LPR;
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int sl = lane & (LPR - 1);
+  const int64_t slot =
+      (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6)) * RPW + lane / LPR;
+  if (slot >= a.n_slots) return;  // a slot leaves as a whole; cross-lane reads never leave the slot
+  const int tile = static_cast<int>(slot / a.n_rows);
+  const int i = static_cast<int>(slot - static_cast<int64_t>(tile) * a.n_rows);
+  const int row = a.row_order ? a.row_order[i] : i;
+  const int f0 = tile * TW + sl * VEC;
+  const bool fok = f0 < a.F;  // lanes past the end of a partial last tile only take part in the cross-lane reads
+  const int head = (MH && fok) ? f0 / a.D : 0;
+  const int64_t F = a.F;
+  const float *fp = a.feat + f0;
+  const float *wp = a.w + head;
+  int e = a.indptr[row];
+  const int end = a.indptr[row + 1];
+  V acc = vzero<VEC>();
+  for (; e < end; e += LPR) {
+    const int n = min(LPR, end - e);
+    int my_col = 0;
+    float my_val = 0.0f;
+    if (sl < n) {
+      my_col = a.indices[e + sl];
+      if (!MH) my_val = a.w[e + sl];
+    }
+    int j = 0;
+    for (; j + U <= n; j += U) {
+      V x[U];
+      float v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int c = slot_read<LPR>(my_col, j + u, lane);
+        x[u] = fok ? *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F) : vzero<VEC>();
+        if (MH)
+          v[u] = wp[static_cast<int64_t>(e + j + u) * a.H];
+        else
+          v[u] = __int_as_float(slot_read<LPR>(__float_as_int(my_val), j + u, lane));
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) axpy(acc, v[u], x[u]);
+    }
+    for (; j < n; ++j) {
+      const int c = slot_read<LPR>(my_col, j, lane);
+      const V x = fok ? *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F) : vzero<VEC>();
+      float v;
+      if (MH)
+        v = wp[static_cast<int64_t>(e + j) * a.H];
+      else
+        v = __int_as_float(slot_read<LPR>(__float_as_int(my_val), j, lane));
+      axpy(acc, v, x);
+    }
+  }
+  if (fok) *reinterpret_cast<V *>(a.out + static_cast<int64_t>(row) * F + f0) = acc;
+}
+
+// Wave-per-(row, tile) kernel (LPR = 64): the row bounds and each neighbour's
+// column id and value live in scalar registers, so a gather is one vector load
+// from a scalar base plus the lane's fixed offset, with no per-lane address
+// arithmetic.
+template <int VEC, int U, bool MH>
+__global__ __launch_bounds__(kBlockThreads) void spmm_wave_kernel(const SpmmArgs a) {
+  using V = typename VecOf<VEC>::type;
+  constexpr int TW = VEC * kWaveSize;
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int64_t slot = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+  if (slot >= a.n_slots) return;
+  const int tile = __builtin_amdgcn_readfirstlane(static_cast<int>(slot / a.n_rows));
+  const int i = __builtin_amdgcn_readfirstlane(static_cast<int>(slot - static_cast<int64_t>(tile) * a.n_rows));
+  const int row = __builtin_amdgcn_readfirstlane(a.row_order ? a.row_order[i] : i);
+  const int f0 = tile * TW + lane * VEC;
+  const bool fok = f0 < a.F;
+  const int head = (MH && fok) ? f0 / a.D : 0;
+  const int64_t F = a.F;
+  const float *fp = a.feat + f0;
+  const float *wp = a.w + head;
+  int e = __builtin_amdgcn_readfirstlane(a.indptr[row]);
+  const int end = __builtin_amdgcn_readfirstlane(a.indptr[row + 1]);
+  V acc = vzero<VEC>();
+  for (; e < end; e += kWaveSize) {
+    const int n = min(kWaveSize, end - e);
+    int my_col = 0;
+    float my_val = 0.0f;
+    if (lane < n) {
+      my_col = a.indices[e + lane];
+      if (!MH) my_val = a.w[e + lane];
+    }
+    int j = 0;
+    for (; j + U <= n; j += U) {
+      V x[U];
+      float v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int c = __builtin_amdgcn_readlane(my_col, j + u);
+        x[u] = fok ? *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F) : vzero<VEC>();
+        if (MH)
+          v[u] = wp[static_cast<int64_t>(e + j + u) * a.H];
+        else
+          v[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_val), j + u));
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) axpy(acc, v[u], x[u]);
+    }
+    for (; j < n; ++j) {
+      const int c = __builtin_amdgcn_readlane(my_col, j);
+      const V x = fok ? *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F) : vzero<VEC>();
+      float v;
+      if (MH)
+        v = wp[static_cast<int64_t>(e + j) * a.H];
+      else
+        v = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_val), j));
+      axpy(acc, v, x);
+    }
+  }
+  if (fok) *reinterpret_cast<V *>(a.out + static_cast<int64_t>(row) * F + f0) = acc;
+}
+
+template <int VEC, int LPR, int U>
+int launch_slot(const SpmmArgs &a, hipStream_t stream) {
+  constexpr int RPW = kWaveSize / LPR;
+  const int64_t waves = (a.n_slots + RPW - 1) / RPW;
+  const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
+  if (blocks > 0x7fffffffLL) return fail(FG_EUNSUPPORTED, "SpMM launch needs %lld blocks", (long long)blocks);
+  if (a.H > 1)
+    spmm_slot_kernel<VEC, LPR, U, true><<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(a);
+  else
+    spmm_slot_kernel<VEC, LPR, U, false><<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(a);
+  FG_HIP_TRY(hipGetLastError());
+  return FG_OK;
+}
+
+template <int VEC, int U>
+int launch_wave(const SpmmArgs &a, hipStream_t stream) {
+  const int64_t blocks = (a.n_slots + kWavesPerBlock - 1) / kWavesPerBlock;
+  if (blocks > 0x7fffffffLL) return fail(FG_EUNSUPPORTED, "SpMM launch needs %lld blocks", (long long)blocks);
+  if (a.H > 1)
+    spmm_wave_kernel<VEC, U, true><<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(a);
+  else
+    spmm_wave_kernel<VEC, U, false><<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(a);
+  FG_HIP_TRY(hipGetLastError());
+  return FG_OK;
+}
+
+template <int VEC, int LPR>
+int dispatch_unroll(const SpmmArgs &a, const SpmmShape &s, hipStream_t stream) {
+  if (LPR == kWaveSize && s.scalar_path) {
+    switch (s.unroll) {
+      case 4: return launch_wave<VEC, 4>(a, stream);
+      case 8: return launch_wave<VEC, 8>(a, stream);
+      case 16: return launch_wave<VEC, 16>(a, stream);
+    }
+  } else {
+    switch (s.unroll) {
+      case 4: return launch_slot<VEC, LPR, 4>(a, stream);
+      case 8: return launch_slot<VEC, LPR, 8>(a, stream);
+      case 16: return launch_slot<VEC, LPR, 16>(a, stream);
+    }
+  }
+  return fail(FG_EINVAL, "spmm unroll %d is not one of 4, 8, 16", s.unroll);
+}
+
+template <int VEC>
+int dispatch_lpr(const SpmmArgs &a, const SpmmShape &s, hipStream_t stream) {
+  switch (s.lpr) {
+    case 8: return dispatch_unroll<VEC, 8>(a, s, stream);
+    case 16: return dispatch_unroll<VEC, 16>(a, s, stream);
+    case 32: return dispatch_unroll<VEC, 32>(a, s, stream);
+    case 64: return dispatch_unroll<VEC, 64>(a, s, stream);
+  }
+  return fail(FG_EINVAL, "spmm lanes per row slot %d is not one of 8, 16, 32, 64", s.lpr);
+}
+
+}  // namespace
+
+// Widest per-lane vector that the feature length, the head length and the
+// base addresses allow.
+static int spmm_max_vec(const SpmmArgs &a) {
+  if (a.D % 4 == 0 && aligned_to(a.feat, 16) && aligned_to(a.out, 16)) return 4;
+  if (a.D % 2 == 0 && aligned_to(a.feat, 8) && aligned_to(a.out, 8)) return 2;
+  return 1;
+}
+
+SpmmShape spmm_choose_shape(const SpmmArgs &a, int feat_tiles) {
+  const Config &cfg = config();
+  SpmmShape s;
+  const int max_vec = spmm_max_vec(a);
+  s.vec = (cfg.spmm_vec > 0 && cfg.spmm_vec <= max_vec) ? cfg.spmm_vec : max_vec;
+  // tile width asked for: the whole row, or about F / feat_tiles floats
+  int want = a.F;
+  if (feat_tiles > 1) want = (a.F + feat_tiles - 1) / feat_tiles;
+  int lanes = pow2_ceil((want + s.vec - 1) / s.vec);
+  if (lanes < 8) lanes = 8;
+  if (lanes > kWaveSize) lanes = kWaveSize;
+  s.lpr = cfg.spmm_lpr > 0 ? cfg.spmm_lpr : lanes;
+  s.unroll = cfg.spmm_unroll > 0 ? cfg.spmm_unroll : 8;
+  s.scalar_path = cfg.spmm_scalar_path >= 0 ? cfg.spmm_scalar_path : 0;
+  if (s.lpr != kWaveSize) s.scalar_path = 0;
+  return s;
+}
+
+int spmm_launch(const SpmmArgs &a, const SpmmShape &s, hipStream_t stream) {
+  if (a.n_slots == 0) return FG_OK;
+  switch (s.vec) {
+    case 1: return dispatch_lpr<1>(a, s, stream);
+    case 2: return dispatch_lpr<2>(a, s, stream);
+    case 4: return dispatch_lpr<4>(a, s, stream);
+  }
+  return fail(FG_EINVAL, "spmm floats per lane %d is not one of 1, 2, 4", s.vec);
+}
+
+}  // namespace fg

@@ -1,0 +1,179 @@
+"""SDDMM module classes on the HIP target.
+
+Same call surface as the reference's featgraph.module.sddmm (SDDMMbase
+module/sddmm.py:11-165, VanillaSDDMMcuda :179-187).  Operand naming follows the
+reference's tests, not its docstring: SrcFeat has one row per COLUMN of the
+adjacency matrix and DstFeat one per ROW (tests/test_module_sddmm.py:18-19,
+op/vanilla_sddmm.py:47).
+"""
+import ctypes
+
+import numpy as np
+import torch
+
+from .. import _lib
+from ..runtime import NDArray, hip
+from . import _common as C
+
+
+def normalize_coo(adj_scipy):
+    """COO view of the input with int32 row / col arrays (host side); module/sddmm.py:28-33, :51-52.
+    Edge values are never read.  Returns (row, col, shape)."""
+    if not hasattr(adj_scipy, "format"):
+        raise TypeError("adjacency must be a scipy sparse matrix, got %s" % type(adj_scipy).__name__)
+    coo = adj_scipy if adj_scipy.format == "coo" else adj_scipy.tocoo()
+    num_rows, num_cols = coo.shape
+    row = C.to_int32_index(coo.row, "row")
+    col = C.to_int32_index(coo.col, "col")
+    if row.shape[0] != col.shape[0]:
+        raise ValueError("row and col differ in length")  # op/vanilla_sddmm.py:40
+    C.check_index_range(row, num_rows, "row")
+    C.check_index_range(col, num_cols, "col")
+    return row, col, (num_rows, num_cols)
+
+
+class SDDMMbase:
+    """Base class of the SDDMM-like modules (reference: module/sddmm.py:11-165)."""
+
+    def __init__(self, adj_scipy, num_row_partitions=1, num_col_partitions=1):
+        assert num_row_partitions >= 1, "num_row_partitions should be larger than or equal to 1"
+        assert num_col_partitions >= 1, "num_col_partitions should be larger than or equal to 1"
+        if num_row_partitions != 1 or num_col_partitions != 1:
+            raise NotImplementedError("2-D graph partitioning is a CPU cache-blocking scheme of the x86 target; "
+                                      "the HIP target takes no partition counts")
+        row, col, (self._num_rows, self._num_cols) = normalize_coo(adj_scipy)
+        self._num_row_partitions = 1
+        self._num_col_partitions = 1
+        self._nnz = int(row.shape[0])
+        self._target = None
+        self._ctx = None
+        self._register()
+        C.require_device()
+        self._adj_row_dev = torch.from_numpy(row).to(self._ctx)  # one upload per module (module/sddmm.py:59-60)
+        self._adj_col_dev = torch.from_numpy(col).to(self._ctx)
+        self._built = False
+        self.out_tvm = None
+
+    def _register(self):
+        raise NotImplementedError("Please register target and ctx.")
+
+    def _heads_and_len(self, feat_shape):
+        if len(feat_shape) != 2:
+            raise ValueError("features must be 2-D [num_vertices, feat_len], got %s" % (feat_shape,))
+        return 1, int(feat_shape[1])
+
+    def _parse_build(self, input_placeholders, compute_args, schedule_args):
+        compute_args = C.check_known_keys(compute_args, ("num_feat_partitions",), "compute_args")
+        schedule_args = C.check_known_keys(
+            schedule_args, ("num_feat_partitions", "num_cuda_blocks", "num_threads_per_cuda_block"), "schedule_args")
+        for args in (compute_args, schedule_args):
+            # feature tiling needs a cross-block reduction on a GPU; the reference's CUDA schedules
+            # refuse it too (op/vanilla_sddmm.py:79-80)
+            assert args.get("num_feat_partitions", 1) in (None, 0, 1), \
+                "the GPU schedule for sddmm does not support feat dimension tiling"
+        if len(input_placeholders) != 2:
+            raise ValueError("expected placeholders [SrcFeat, DstFeat]")
+        for p in input_placeholders:
+            if str(p.dtype) != "float32":
+                raise TypeError("operands must be float32, got %s" % p.dtype)
+        src_shape, dst_shape = (tuple(int(s) for s in p.shape) for p in input_placeholders)
+        assert src_shape[1:] == dst_shape[1:], "dimension mismatch"  # op/vanilla_sddmm.py:38
+        if src_shape[0] != self._num_cols:
+            raise ValueError("SrcFeat has %d rows, the adjacency matrix %d columns" % (src_shape[0], self._num_cols))
+        if dst_shape[0] != self._num_rows:
+            raise ValueError("DstFeat has %d rows, the adjacency matrix %d rows" % (dst_shape[0], self._num_rows))
+        H, D = self._heads_and_len(src_shape)
+        if H * D < 1:
+            raise ValueError("feature length must be positive")
+        return [src_shape, dst_shape], H, D
+
+    def build(self, input_placeholders, compute_args, schedule_args):
+        """Fix operand shapes and allocate the (zero-filled, reused) output: module/sddmm.py:72-92.
+        The reference's CUDA launch keys in schedule_args are accepted and ignored."""
+        shapes, H, D = self._parse_build(input_placeholders, compute_args, schedule_args)
+        self._input_shapes = shapes
+        self._H, self._D = H, D
+        out_shape = (self._nnz,) if len(shapes[0]) == 2 else (self._nnz, H)
+        self.out_tvm = NDArray(torch.zeros(out_shape, dtype=torch.float32, device=self._ctx))
+        self._built = True
+
+    def lower_to_ir(self, input_placeholders, compute_args, schedule_args):
+        """Description of the launch (module/sddmm.py:94-113 returns TVM IR)."""
+        _, H, D = self._parse_build(input_placeholders, compute_args, schedule_args)
+        buf = ctypes.create_string_buffer(1024)
+        _lib.check(_lib.lib().fg_sddmm_describe(self._nnz, H, D, buf, len(buf)))
+        return buf.value.decode()
+
+    def _launch(self, tensors):
+        src, dst = tensors
+        _lib.check(_lib.lib().fg_sddmm_coo_mh_f32(
+            self._nnz, self._adj_row_dev.data_ptr(), self._adj_col_dev.data_ptr(), src.data_ptr(), dst.data_ptr(),
+            self.out_tvm.tensor.data_ptr(), self._H, self._D, C.current_stream_handle(self._ctx)))
+
+    def _checked_inputs(self, input_ndarrays):
+        if not self._built:
+            raise RuntimeError("call build() before run()")
+        if len(input_ndarrays) != 2:
+            raise ValueError("expected input arrays [src_feat, dst_feat]")
+        return [C.check_operand(x, s, self._ctx, n)
+                for x, s, n in zip(input_ndarrays, self._input_shapes, ("SrcFeat", "DstFeat"))]
+
+    def run(self, input_tvm_ndarrays):
+        """Enqueue the kernel and return the module-owned output (one float per edge,
+        in the order of the adjacency's row / col arrays): module/sddmm.py:115-129."""
+        tensors = self._checked_inputs(input_tvm_ndarrays)
+        with torch.cuda.device(self._ctx):
+            self._launch(tensors)
+        return self.out_tvm
+
+    def measure_average_time(self, input_tvm_ndarrays, num_runs):
+        """Average seconds per run over num_runs runs after one warm-up (module/sddmm.py:131-150)."""
+        tensors = self._checked_inputs(input_tvm_ndarrays)
+        with torch.cuda.device(self._ctx):
+            return C.time_calls(lambda: self._launch(tensors), self._ctx, num_runs)
+
+    @property
+    def edge_mapping(self):
+        # module/sddmm.py:152-157: only the partitioned x86 path has one
+        assert self._target not in ("cuda", "hip"), "no graph partitioning on %s, no edge_mapping" % self._target
+        assert self._num_row_partitions > 1 or self._num_col_partitions > 1, \
+            "no graph partitioning, no edge_mapping"
+        return None
+
+    @property
+    def ctx(self):
+        return self._ctx
+
+    @property
+    def target(self):
+        return self._target
+
+
+class VanillaSDDMMhip(SDDMMbase):
+    """COO SDDMM on the GPU; constructor signature of VanillaSDDMMcuda (module/sddmm.py:179-181)."""
+
+    def __init__(self, adj_scipy):
+        super().__init__(adj_scipy, num_row_partitions=1, num_col_partitions=1)
+
+    def _register(self):
+        self._target = "hip"
+        self._ctx = hip(0)
+
+
+class MultiHeadSDDMMhip(SDDMMbase):
+    """Per-head dot products (GAT attention scores): Out[e,h] = sum_d Src[col[e],h,d] * Dst[row[e],h,d].
+
+    Not in the reference; operands are [num_vertices, H, D], the output [nnz, H].
+    """
+
+    def __init__(self, adj_scipy):
+        super().__init__(adj_scipy, num_row_partitions=1, num_col_partitions=1)
+
+    def _register(self):
+        self._target = "hip"
+        self._ctx = hip(0)
+
+    def _heads_and_len(self, feat_shape):
+        if len(feat_shape) != 3:
+            raise ValueError("features must be 3-D [num_vertices, num_heads, head_len], got %s" % (feat_shape,))
+        return int(feat_shape[1]), int(feat_shape[2])

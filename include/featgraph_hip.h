@@ -1,0 +1,141 @@
+/*
+ * C ABI of libfeatgraph_hip.so: FeatGraph's vanilla CSR SpMM and COO SDDMM
+ * (and their multi-head forms) as hand-written HIP kernels for gfx950.
+ *
+ * These entry points take the place of the functions that the reference
+ * obtains from tvm.build and then calls with positional device arrays:
+ *   SpMM  : module/spmm.py:108-109 (build) and :159-160 (call), argument order
+ *           (SrcFeat, indptr, indices, vals, Out);
+ *   SDDMM : module/sddmm.py:89-90 (build) and :128 (call), argument order
+ *           (SrcFeat, DstFeat, row, col, Out).
+ *
+ * Conventions
+ *   - Every data pointer is DEVICE memory owned by the caller.  The library
+ *     never copies user data between host and device and never allocates or
+ *     frees a caller-visible buffer.  A plan owns only its private row list.
+ *   - Index arrays are int32, values and features float32, row-major, dense.
+ *   - Kernels are enqueued on `stream` (a hipStream_t passed as void*, NULL =
+ *     the default stream) and the call returns without synchronising.
+ *   - Every output element is written by exactly one lane; results are
+ *     deterministic and do not depend on launch shape or tile settings.
+ *   - Return value: FG_OK or a negative FG_E* code; fg_last_error() then holds
+ *     a message (thread-local).  No entry point aborts on bad arguments.
+ *   - Index CONTENTS (column ids within range, monotone indptr) are the
+ *     caller's contract, as they are for the reference's generated kernels;
+ *     fg_spmm_plan_create checks indptr, fg_check_indices checks ids.
+ */
+#ifndef FEATGRAPH_HIP_H_
+#define FEATGRAPH_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FG_API __attribute__((visibility("default")))
+
+#define FG_OK 0
+#define FG_EINVAL (-1)       /* bad argument (null pointer, negative size, shape mismatch) */
+#define FG_EHIP (-2)         /* a HIP runtime call failed; message names it */
+#define FG_ENOMEM (-3)       /* host or device allocation for a plan failed */
+#define FG_EUNSUPPORTED (-4) /* argument combination outside what the kernels cover */
+
+typedef struct fg_spmm_plan fg_spmm_plan;
+
+/* Library version (major*100 + minor). */
+FG_API int fg_version(void);
+
+/* Message of the last failing call on this thread ("" when none). */
+FG_API const char *fg_last_error(void);
+
+/*
+ * Degree-aware row schedule for one CSR adjacency matrix.  Replaces the
+ * per-module preprocessing of SpMMbase.__init__ (module/spmm.py:58-69), which
+ * in the reference only uploads the three CSR arrays.  Reads indptr once
+ * (device to host), checks that it starts at 0, is non-decreasing and ends at
+ * nnz, and stores on the device the row ids sorted by descending degree (ties
+ * by ascending row id).  The plan BORROWS indptr and indices: both must stay
+ * alive and unchanged until fg_spmm_plan_destroy.
+ */
+FG_API int fg_spmm_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr,
+                        const int32_t *indices, fg_spmm_plan **plan);
+FG_API void fg_spmm_plan_destroy(fg_spmm_plan *plan);
+
+/* Copies the plan's row order (n_rows int32) to HOST memory at row_order_host
+ * and, when non-null, the largest row degree to *max_degree. */
+FG_API int fg_spmm_plan_row_order(const fg_spmm_plan *plan, int32_t *row_order_host, int32_t *max_degree);
+
+/*
+ * Out[r, f] = sum over e in [indptr[r], indptr[r+1]) of vals[e] * feat[indices[e], f]
+ * accumulated in float32, sequentially in CSR order from +0, one rounded
+ * multiply and one rounded add per term: the loop nest of
+ * vanilla_spmm_csr_x86 / _cuda (op/vanilla_spmm.py:46-56, :114-123).
+ * feat is [n_cols, F], out is [n_rows, F]; rows without nonzeros become 0.
+ * feat_tiles is the reference's num_feat_partitions (op/vanilla_spmm.py:41):
+ * 0 lets the library choose the feature-tile width, P >= 1 asks for tiles of
+ * about F/P floats.  It changes the launch shape only, never a result bit.
+ */
+FG_API int fg_spmm_csr_f32(const fg_spmm_plan *plan, const float *feat, const float *vals, float *out, int32_t F,
+                    int32_t feat_tiles, void *stream);
+
+/*
+ * Multi-head generalised SpMM (no counterpart in the reference, whose
+ * op/__init__.py:1-5 exports vanilla operators only; same message function as
+ * op/vanilla_spmm.py:46-53 with a per-head weight):
+ * Out[r, h, d] = sum over e in row r of w[e, h] * feat[indices[e], h, d].
+ * feat [n_cols, H, D], w [nnz, H], out [n_rows, H, D].  H = 1 gives
+ * fg_spmm_csr_f32 bit for bit.
+ */
+FG_API int fg_spmm_csr_mh_f32(const fg_spmm_plan *plan, const float *feat, const float *w, float *out, int32_t H,
+                       int32_t D, int32_t feat_tiles, void *stream);
+
+/*
+ * Out[e] = sum_k src[col[e], k] * dst[row[e], k]   (op/vanilla_sddmm.py:43-47;
+ * note src is indexed by COLUMN ids and dst by ROW ids, as the reference's
+ * tests shape them: tests/test_module_sddmm.py:18-19).
+ * src [n_cols, F], dst [n_rows, F], out [nnz].  Any nnz >= 0.
+ */
+FG_API int fg_sddmm_coo_f32(int64_t nnz, const int32_t *row, const int32_t *col, const float *src, const float *dst,
+                     float *out, int32_t F, void *stream);
+
+/*
+ * Multi-head SDDMM (no counterpart in the reference; the edge function of
+ * op/vanilla_sddmm.py:47 per head): Out[e, h] = sum_d src[col[e], h, d] * dst[row[e], h, d].
+ * src [n_cols, H, D], dst [n_rows, H, D], out [nnz, H].  H = 1 gives
+ * fg_sddmm_coo_f32 bit for bit.
+ */
+FG_API int fg_sddmm_coo_mh_f32(int64_t nnz, const int32_t *row, const int32_t *col, const float *src, const float *dst,
+                        float *out, int32_t H, int32_t D, void *stream);
+
+/*
+ * Debug aid: counts entries of idx[0..n) outside [0, bound) on the device and
+ * writes the count to *n_bad (host).  Synchronises `stream`.
+ */
+FG_API int fg_check_indices(int64_t n, const int32_t *idx, int64_t bound, int64_t *n_bad, void *stream);
+
+/*
+ * Launch-shape overrides for tuning and tests.
+ * Keys: "spmm.vec" (floats per lane: 1, 2, 4), "spmm.lpr" (lanes per row
+ * slot: 8, 16, 32, 64), "spmm.unroll" (gathers in flight per lane: 4, 8, 16),
+ * "spmm.scalar_path" (0/1: wave-per-row variant that keeps column ids in
+ * scalar registers), "spmm.sorted" (0/1: visit rows by descending degree or
+ * in natural order), "sddmm.group" (lanes per dot product: 1..16),
+ * "sddmm.batches" (64-edge batches per wave).  Value 0 restores the default of
+ * a size; for the two 0/1 flags a negative value does.
+ * The spmm.* keys change the launch shape only; "sddmm.group" also changes the
+ * shape of the summation tree, i.e. the last bits of an SDDMM result.
+ */
+FG_API int fg_config_set(const char *key, int32_t value);
+FG_API int fg_config_get(const char *key, int32_t *value);
+
+/* Human-readable description of the launch the library would use for a
+ * feature length (the counterpart of lower_to_ir, module/spmm.py:113-140).
+ * Writes at most cap bytes including the terminator. */
+FG_API int fg_spmm_describe(const fg_spmm_plan *plan, int32_t H, int32_t D, int32_t feat_tiles, char *buf, int64_t cap);
+FG_API int fg_sddmm_describe(int64_t nnz, int32_t H, int32_t D, char *buf, int64_t cap);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FEATGRAPH_HIP_H_ */

@@ -1,0 +1,173 @@
+"""GPU parity tests of the SDDMM modules, through the module layer and the C ABI.
+
+Bar: float32 results within rtol=1e-5 / atol=1e-4 of the CPU restatement (whose
+k-order the reference does not pin) and of the float64 closed form; structure
+properties (edge order, duplicates, permutations) hold bit for bit.
+"""
+import numpy as np
+import pytest
+import scipy.sparse
+
+from conftest import reference_test_matrix
+from featgraph_amd import _lib, datasets, nd, placeholder
+from featgraph_amd.module import MultiHeadSDDMMhip, VanillaSDDMMhip
+from oracle import ref
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-5, 1e-4
+
+
+def _run_sddmm(adj, src_np, dst_np, cls=VanillaSDDMMhip, schedule_args=None):
+    module = cls(adj)
+    module.build([placeholder(src_np.shape), placeholder(dst_np.shape)], {}, schedule_args or {})
+    out = module.run([nd.array(src_np, module.ctx), nd.array(dst_np, module.ctx)])
+    return out.asnumpy()
+
+
+@pytest.fixture
+def config_guard():
+    yield
+    _lib.config_set("sddmm.group", 0)
+    _lib.config_set("sddmm.batches", 0)
+
+
+# the reference's own test on its matrix family (tests/test_module_sddmm.py:44-70)
+@pytest.mark.parametrize("num_cuda_blocks", [32, 256])
+def test_vanilla_sddmm_hip_like_the_reference_cuda_test(num_cuda_blocks):
+    coo = reference_test_matrix("coo", seed=0)
+    rng = np.random.default_rng(1)
+    src = rng.random((coo.shape[1], 128)).astype("float32")
+    dst = rng.random((coo.shape[0], 128)).astype("float32")
+    out = _run_sddmm(coo, src, dst, schedule_args={"num_cuda_blocks": num_cuda_blocks})
+    lhs, rhs = src[coo.col], dst[coo.row]
+    np.testing.assert_allclose((lhs * rhs).sum(axis=-1), out, rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(out, ref.sddmm_x86(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(out, ref.sddmm_f64(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("F", [1, 2, 3, 4, 7, 8, 16, 30, 32, 33, 64, 100, 128, 256, 260, 512, 513])
+def test_feature_lengths(F):
+    coo = reference_test_matrix("coo", seed=F)
+    src, dst = datasets.sddmm_operands(coo, F)
+    out = _run_sddmm(coo, src, dst)
+    assert out.shape == (coo.nnz,)
+    np.testing.assert_allclose(out, ref.sddmm_x86(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
+
+
+def test_exact_on_integers_and_operand_roles():
+    coo = reference_test_matrix("coo", seed=3, shape=(90, 41), density=0.3)
+    rng = np.random.default_rng(3)
+    src = rng.integers(-8, 9, (41, 64)).astype(np.float32)        # one row per COLUMN
+    dst = rng.integers(-8, 9, (90, 64)).astype(np.float32)        # one row per ROW
+    want = (src[coo.col].astype(np.int64) * dst[coo.row].astype(np.int64)).sum(-1).astype(np.float32)
+    assert np.array_equal(_run_sddmm(coo, src, dst), want)
+
+
+@pytest.mark.parametrize("F", [32, 64, 128, 512])
+def test_powerlaw_graph_row_sorted_and_shuffled(F):
+    adj = datasets.config_graph("c2-mini")
+    coo = adj.tocoo()
+    src, dst = datasets.sddmm_operands(coo, F)
+    out = _run_sddmm(coo, src, dst)
+    np.testing.assert_allclose(out, ref.sddmm_x86(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
+    perm = np.random.default_rng(4).permutation(coo.nnz)
+    shuffled = scipy.sparse.coo_matrix((coo.data[perm], (coo.row[perm], coo.col[perm])), shape=coo.shape)
+    assert np.array_equal(_run_sddmm(shuffled, src, dst), out[perm])     # edge order is only an order
+
+
+def test_c1_configuration_and_committed_golden():
+    import os
+    adj = datasets.config_graph("c1").tocoo()
+    src, dst = datasets.sddmm_operands(adj, 64)
+    out = _run_sddmm(adj, src, dst)
+    np.testing.assert_allclose(out, ref.sddmm_x86(adj.row, adj.col, src, dst), rtol=RTOL, atol=ATOL)
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "c1_sddmm_f64.npz"))
+    np.testing.assert_allclose(out[gold["edges"]], gold["out_edges"], rtol=RTOL, atol=ATOL)
+
+
+def test_duplicates_tails_and_empty_edge_lists(config_guard):
+    rng = np.random.default_rng(5)
+    src = rng.standard_normal((17, 48), dtype=np.float32)
+    dst = rng.standard_normal((23, 48), dtype=np.float32)
+    for nnz in (1, 63, 64, 65, 255, 257, 1000):
+        row = rng.integers(0, 23, nnz).astype(np.int32)
+        col = rng.integers(0, 17, nnz).astype(np.int32)
+        coo = scipy.sparse.coo_matrix((np.ones(nnz, np.float32), (row, col)), shape=(23, 17))
+        out = _run_sddmm(coo, src, dst)
+        np.testing.assert_allclose(out, ref.sddmm_x86(row, col, src, dst), rtol=RTOL, atol=ATOL)
+        twice = scipy.sparse.coo_matrix((np.ones(2 * nnz, np.float32), (np.tile(row, 2), np.tile(col, 2))), shape=(23, 17))
+        assert np.array_equal(_run_sddmm(twice, src, dst), np.tile(out, 2))
+        for batches in (1, 3):
+            _lib.config_set("sddmm.batches", batches)
+            assert np.array_equal(_run_sddmm(coo, src, dst), out)
+        _lib.config_set("sddmm.batches", 0)
+    empty = scipy.sparse.coo_matrix((23, 17), dtype=np.float32)
+    assert _run_sddmm(empty, src, dst).shape == (0,)
+
+
+def test_swapping_operand_roles_on_the_transpose_gives_the_same_bits():
+    coo = reference_test_matrix("coo", seed=6, shape=(50, 70), density=0.2)
+    src, dst = datasets.sddmm_operands(coo, 96)
+    t = scipy.sparse.coo_matrix((coo.data, (coo.col, coo.row)), shape=(70, 50))     # same edge order, roles swapped
+    assert np.array_equal(_run_sddmm(coo, src, dst), _run_sddmm(t, dst, src))
+
+
+def test_group_sizes_agree_within_rounding(config_guard):
+    coo = reference_test_matrix("coo", seed=7)
+    src, dst = datasets.sddmm_operands(coo, 64)
+    want = ref.sddmm_f64(coo.row, coo.col, src, dst)
+    for g in (1, 2, 4, 8, 16):
+        _lib.config_set("sddmm.group", g)
+        np.testing.assert_allclose(_run_sddmm(coo, src, dst), want, rtol=RTOL, atol=ATOL)
+
+
+def test_module_surface(adj_127x255):
+    coo = adj_127x255.tocoo()
+    module = VanillaSDDMMhip(coo)
+    assert module.target == "hip"
+    with pytest.raises(AssertionError):
+        module.edge_mapping                                           # module/sddmm.py:152-157
+    with pytest.raises(AssertionError):
+        module.build([placeholder((coo.shape[1], 8)), placeholder((coo.shape[0], 8))], {"num_feat_partitions": 2}, {})
+    with pytest.raises(AssertionError):
+        module.build([placeholder((coo.shape[1], 8)), placeholder((coo.shape[0], 16))], {}, {})
+    module.build([placeholder((coo.shape[1], 8)), placeholder((coo.shape[0], 8))], {}, {})
+    assert np.all(module.out_tvm.asnumpy() == 0) and module.out_tvm.shape == (coo.nnz,)
+    src, dst = datasets.sddmm_operands(coo, 8)
+    a = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)])
+    b = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)])
+    assert a is b is module.out_tvm
+    t = module.measure_average_time([nd.array(src, module.ctx), nd.array(dst, module.ctx)], 3)
+    assert isinstance(t, float) and 0 < t < 1.0
+    with pytest.raises(ValueError):
+        module.run([nd.array(dst, module.ctx), nd.array(src, module.ctx)])              # roles swapped: shapes differ
+
+
+# ---------------------------------------------------------------- multi-head
+@pytest.mark.parametrize("H,D", [(8, 16), (8, 32), (8, 64), (3, 5), (2, 130), (1, 64), (5, 4)])
+def test_multihead_sddmm_matches_closed_form(H, D):
+    coo = datasets.config_graph("c4-mini").tocoo()
+    src, dst = datasets.sddmm_operands(coo, (H, D))
+    out = _run_sddmm(coo, src, dst, cls=MultiHeadSDDMMhip)
+    assert out.shape == (coo.nnz, H)
+    np.testing.assert_allclose(out, ref.sddmm_mh(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
+    want = np.einsum("ehd,ehd->eh", src[coo.col].astype(np.float64), dst[coo.row].astype(np.float64))
+    np.testing.assert_allclose(out, want, rtol=RTOL, atol=ATOL)
+
+
+def test_multihead_sddmm_with_one_head_is_the_vanilla_kernel():
+    coo = datasets.config_graph("c4-mini").tocoo()
+    src, dst = datasets.sddmm_operands(coo, (1, 64))
+    mh = _run_sddmm(coo, src, dst, cls=MultiHeadSDDMMhip)
+    assert np.array_equal(mh[:, 0], _run_sddmm(coo, src[:, 0], dst[:, 0]))
+
+
+def test_each_head_is_a_vanilla_sddmm_on_its_slice():
+    coo = datasets.config_graph("c4-mini").tocoo()
+    H, D = 8, 64
+    src, dst = datasets.sddmm_operands(coo, (H, D))
+    mh = _run_sddmm(coo, src, dst, cls=MultiHeadSDDMMhip)
+    for h in (0, 5):
+        one = _run_sddmm(coo, np.ascontiguousarray(src[:, h]), np.ascontiguousarray(dst[:, h]))
+        assert np.array_equal(mh[:, h], one)

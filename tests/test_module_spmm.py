@@ -1,0 +1,258 @@
+"""GPU parity tests of the SpMM modules, through the module layer and the C ABI.
+
+Bar: float32 results equal the CPU restatement of the reference's x86 loop nest
+BIT FOR BIT (the kernel keeps its summation order and rounding), which implies
+the stated tolerance rtol=1e-5 / atol=1e-4; scipy's csr.dot is checked as the
+reference's own tests do (tests/test_module_spmm.py:29-30, rtol=atol=1e-4).
+"""
+import numpy as np
+import pytest
+import scipy.sparse
+
+from conftest import reference_test_matrix
+from featgraph_amd import _lib, datasets, nd, placeholder
+from featgraph_amd.module import MultiHeadSpMMhip, VanillaSpMMhip
+from oracle import ref
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-5, 1e-4   # the tolerance the project states for float32 results
+
+
+def _run_spmm(adj, feat_np, compute_args=None, schedule_args=None):
+    module = VanillaSpMMhip(adj)
+    SrcFeat = placeholder((adj.shape[1], feat_np.shape[1]))
+    module.build([SrcFeat], compute_args or {}, schedule_args or {})
+    src_feat = nd.array(feat_np, module.ctx)
+    return module.run([src_feat]).asnumpy()
+
+
+def _oracle(adj, feat_np, P=1):
+    csr = adj.tocsr() if adj.format != "csr" else adj
+    return ref.spmm_csr_x86(csr.indptr, csr.indices, csr.data.astype(np.float32), feat_np, P)
+
+
+@pytest.fixture
+def config_guard():
+    yield
+    for key in ("spmm.vec", "spmm.lpr", "spmm.unroll"):
+        _lib.config_set(key, 0)
+    for key in ("spmm.scalar_path", "spmm.sorted"):
+        _lib.config_set(key, -1)
+
+
+# the reference's own test, on its matrix family (tests/test_module_spmm.py:37-59)
+@pytest.mark.parametrize("num_threads_per_cuda_block", [32, 128, None])
+def test_vanilla_spmm_hip_like_the_reference_cuda_test(adj_127x255, num_threads_per_cuda_block):
+    adj = adj_127x255
+    feat = np.random.default_rng(1).random((adj.shape[1], 128)).astype("float32")
+    out = _run_spmm(adj, feat, {}, {"num_threads_per_cuda_block": num_threads_per_cuda_block})
+    np.testing.assert_allclose(adj.dot(feat), out, rtol=1e-4, atol=1e-4)
+    assert np.array_equal(out, _oracle(adj, feat))
+
+
+# ... and its x86 test's feature-partition arguments (:32-34)
+@pytest.mark.parametrize("num_feat_partitions", [1, 4, 8])
+def test_feature_partitions_never_change_a_bit(adj_127x255, num_feat_partitions):
+    adj = adj_127x255
+    feat = np.random.default_rng(2).standard_normal((adj.shape[1], 128), dtype=np.float32)
+    out = _run_spmm(adj, feat, {"num_feat_partitions": num_feat_partitions})
+    assert np.array_equal(out, _oracle(adj, feat, num_feat_partitions))
+
+
+@pytest.mark.parametrize("F", [1, 2, 3, 4, 7, 8, 16, 30, 32, 33, 64, 100, 128, 256, 260, 512, 513, 1024])
+def test_feature_lengths(adj_127x255, F):
+    adj = adj_127x255
+    feat = np.random.default_rng(F).standard_normal((adj.shape[1], F), dtype=np.float32)
+    assert np.array_equal(_run_spmm(adj, feat), _oracle(adj, feat))
+
+
+def test_c1_configuration_and_committed_golden():
+    import hashlib, os
+    adj = datasets.config_graph("c1")
+    feat = datasets.spmm_operands(adj, 64)
+    out = _run_spmm(adj, feat)
+    want = _oracle(adj, feat)
+    assert np.array_equal(out, want)
+    np.testing.assert_allclose(out, ref.spmm_csr_f64(adj.indptr, adj.indices, adj.data, feat), rtol=RTOL, atol=ATOL)
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "c1_spmm.npz"))
+    assert hashlib.sha256(out.tobytes()).hexdigest() == str(gold["sha256"])
+    assert np.array_equal(out[gold["rows"]], gold["out_rows"])
+
+
+@pytest.mark.parametrize("F", [32, 64, 128, 512])
+def test_powerlaw_graph_with_hub_rows(F):
+    adj = datasets.config_graph("c2-mini")
+    feat = datasets.spmm_operands(adj, F)
+    out = _run_spmm(adj, feat)
+    assert np.array_equal(out, _oracle(adj, feat))
+    np.testing.assert_allclose(out, _oracle(adj, feat, 4), rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("key,values", [("spmm.vec", [1, 2, 4]), ("spmm.lpr", [8, 16, 32, 64]),
+                                        ("spmm.unroll", [4, 8, 16]), ("spmm.scalar_path", [0, 1]),
+                                        ("spmm.sorted", [0, 1])])
+@pytest.mark.parametrize("F", [64, 200])
+def test_every_launch_shape_gives_the_same_bits(config_guard, key, values, F):
+    adj = datasets.config_graph("c2-mini")
+    feat = datasets.spmm_operands(adj, F)
+    want = _oracle(adj, feat)
+    for v in values:
+        if key == "spmm.scalar_path":
+            _lib.config_set("spmm.lpr", 64)
+        _lib.config_set(key, v)
+        assert np.array_equal(_run_spmm(adj, feat), want), "%s=%d" % (key, v)
+
+
+@pytest.mark.parametrize("vec", [1, 2, 4])
+@pytest.mark.parametrize("unroll", [4, 16])
+def test_scalar_path_variants(config_guard, vec, unroll):
+    adj = datasets.config_graph("c2-mini")
+    feat = datasets.spmm_operands(adj, 256)
+    _lib.config_set("spmm.lpr", 64)
+    _lib.config_set("spmm.scalar_path", 1)
+    _lib.config_set("spmm.vec", vec)
+    _lib.config_set("spmm.unroll", unroll)
+    assert np.array_equal(_run_spmm(adj, feat), _oracle(adj, feat))
+
+
+def test_summation_order_and_unfused_rounding_on_the_gpu():
+    # the two hand-computed cases that pin the oracle (tests/test_oracle.py), now on the kernel
+    indptr = np.array([0, 4, 8, 10], dtype=np.int32)
+    indices = np.array([0, 1, 2, 3, 3, 2, 1, 0, 4, 5], dtype=np.int32)
+    v = np.float32(1 + 2.0 ** -12)
+    vals = np.array([1, 1, 1, 1, 1, 1, 1, 1, 1, v], dtype=np.float32)
+    feat = np.array([[1e8], [1.0], [-1e8], [1.0], [-(1 + 2.0 ** -11)], [v]], dtype=np.float32)
+    adj = scipy.sparse.csr_matrix((vals, indices, indptr), shape=(3, 6))
+    out = _run_spmm(adj, np.repeat(feat, 8, axis=1))
+    assert np.all(out[0] == 1.0) and np.all(out[1] == 0.0) and np.all(out[2] == 0.0)
+
+
+def test_empty_rows_empty_matrix_and_odd_structures():
+    rng = np.random.default_rng(7)
+    # rows without nonzeros become +0 even though the output buffer is reused
+    indptr = np.array([0, 0, 3, 3, 3, 5, 5], dtype=np.int32)
+    indices = np.array([2, 0, 2, 1, 1], dtype=np.int32)            # unsorted and duplicated columns
+    vals = rng.random(5, dtype=np.float32)
+    adj = scipy.sparse.csr_matrix((vals, indices, indptr), shape=(6, 3))
+    feat = rng.standard_normal((3, 20), dtype=np.float32)
+    module = VanillaSpMMhip(adj)
+    module.build([placeholder((3, 20))], {}, {})
+    module.out_tvm.tensor.fill_(7.0)
+    out = module.run([nd.array(feat, module.ctx)]).asnumpy()
+    assert np.array_equal(out, ref.spmm_csr_x86(indptr, indices, vals, feat))
+    assert np.all(out[[0, 2, 3, 5]] == 0) and not np.signbit(out[0]).any()
+    empty = scipy.sparse.csr_matrix((5, 4), dtype=np.float32)
+    assert np.array_equal(_run_spmm(empty, np.ones((4, 6), dtype=np.float32)), np.zeros((5, 6), dtype=np.float32))
+
+
+def test_single_long_row_and_wide_matrix():
+    rng = np.random.default_rng(8)
+    n_cols = 5000
+    cols = rng.integers(0, n_cols, 9001).astype(np.int32)
+    adj = scipy.sparse.csr_matrix((rng.random(9001, dtype=np.float32), cols, np.array([0, 9001], dtype=np.int32)),
+                                  shape=(1, n_cols))
+    feat = rng.standard_normal((n_cols, 96), dtype=np.float32)
+    out = _run_spmm(adj, feat)
+    assert np.array_equal(out, ref.spmm_csr_x86(adj.indptr, adj.indices, adj.data, feat))
+
+
+def test_row_plan_is_a_stable_sort_by_descending_degree():
+    adj = datasets.config_graph("c2-mini")
+    module = VanillaSpMMhip(adj)
+    order, max_deg = module.row_order()
+    deg = np.diff(adj.indptr)
+    assert np.array_equal(order, np.argsort(-deg.astype(np.int64), kind="stable").astype(np.int32))
+    assert max_deg == deg.max()
+    assert "by-descending-degree" in module.lower_to_ir([placeholder((adj.shape[1], 64))], {}, {})
+
+
+def test_output_is_allocated_once_and_reused(adj_127x255):
+    adj = adj_127x255
+    module = VanillaSpMMhip(adj)
+    module.build([placeholder((adj.shape[1], 32))], {}, {})
+    assert module.target == "hip" and module.out_tvm.shape == (adj.shape[0], 32)
+    assert np.all(module.out_tvm.asnumpy() == 0)                      # zero-filled at build (module/spmm.py:110-111)
+    rng = np.random.default_rng(9)
+    a, b = (rng.standard_normal((adj.shape[1], 32), dtype=np.float32) for _ in range(2))
+    out1 = module.run([nd.array(a, module.ctx)])
+    first = out1.asnumpy()
+    out2 = module.run([nd.array(b, module.ctx)])
+    assert out1 is out2 is module.out_tvm                            # same object, overwritten (module/spmm.py:161)
+    assert np.array_equal(first, _oracle(adj, a)) and np.array_equal(out2.asnumpy(), _oracle(adj, b))
+    t = module.measure_average_time([nd.array(b, module.ctx)], 3)
+    assert isinstance(t, float) and 0 < t < 1.0                      # seconds
+    assert np.array_equal(module.out_tvm.asnumpy(), _oracle(adj, b))
+
+
+def test_argument_errors(adj_127x255):
+    import torch
+    adj = adj_127x255
+    module = VanillaSpMMhip(adj)
+    with pytest.raises(RuntimeError):
+        module.run([nd.array(np.zeros((adj.shape[1], 8), np.float32), module.ctx)])      # before build
+    with pytest.raises(ValueError):
+        module.build([placeholder((adj.shape[1] + 1, 8))], {}, {})
+    with pytest.raises(ValueError):
+        module.build([placeholder((adj.shape[1], 10))], {"num_feat_partitions": 4}, {})   # op/vanilla_spmm.py:41
+    with pytest.raises(TypeError):
+        module.build([placeholder((adj.shape[1], 8))], {"feat_partitions": 2}, {})
+    module.build([placeholder((adj.shape[1], 8))], {}, {})
+    with pytest.raises(ValueError):
+        module.run([nd.array(np.zeros((adj.shape[1], 9), np.float32), module.ctx)])
+    with pytest.raises(TypeError):
+        module.run([nd.array(np.zeros((adj.shape[1], 8), np.float64), module.ctx)])
+    with pytest.raises(ValueError):
+        module.run([torch.zeros((adj.shape[1], 8), dtype=torch.float32)])                  # host tensor
+    with pytest.raises(ValueError):
+        module.run([torch.zeros((8, adj.shape[1]), dtype=torch.float32, device=module.ctx).t()])  # not contiguous
+    with pytest.raises(TypeError):
+        module.run([np.zeros((adj.shape[1], 8), np.float32)])
+
+
+def test_index_check_entry_point():
+    import ctypes, torch
+    idx = torch.tensor([0, 5, -1, 9, 10, 3], dtype=torch.int32, device="cuda")
+    n_bad = ctypes.c_int64(-1)
+    _lib.check(_lib.lib().fg_check_indices(idx.numel(), idx.data_ptr(), 10, ctypes.byref(n_bad), None))
+    assert n_bad.value == 2
+
+
+# ---------------------------------------------------------------- multi-head
+def _run_mh(adj, feat, w, compute_args=None):
+    module = MultiHeadSpMMhip(adj)
+    module.build([placeholder(feat.shape), placeholder(w.shape)], compute_args or {}, {})
+    return module.run([nd.array(feat, module.ctx), nd.array(w, module.ctx)]).asnumpy()
+
+
+@pytest.mark.parametrize("H,D", [(8, 64), (8, 16), (3, 5), (1, 64), (2, 130)])
+def test_multihead_spmm_matches_closed_form(H, D):
+    adj = datasets.config_graph("c4-mini")
+    feat = datasets.spmm_operands(adj, (H, D))
+    w = datasets.softmax_edge_weights(adj, H)
+    out = _run_mh(adj, feat, w)
+    assert out.shape == (adj.shape[0], H, D)
+    assert np.array_equal(out, ref.spmm_mh(adj.indptr, adj.indices, w, feat))
+
+
+def test_multihead_spmm_with_one_head_is_the_vanilla_kernel(config_guard):
+    adj = datasets.config_graph("c4-mini")
+    feat = datasets.spmm_operands(adj, (1, 64))
+    vanilla = _run_spmm(adj, feat[:, 0])
+    for lpr in (16, 64):
+        _lib.config_set("spmm.lpr", lpr)
+        assert np.array_equal(_run_mh(adj, feat, adj.data.reshape(-1, 1).copy())[:, 0], vanilla)
+
+
+@pytest.mark.parametrize("key,values", [("spmm.vec", [1, 2, 4]), ("spmm.lpr", [8, 32, 64]), ("spmm.scalar_path", [1])])
+def test_multihead_launch_shapes_give_the_same_bits(config_guard, key, values):
+    adj = datasets.config_graph("c4-mini")
+    H, D = 8, 32
+    feat = datasets.spmm_operands(adj, (H, D))
+    w = datasets.softmax_edge_weights(adj, H)
+    want = ref.spmm_mh(adj.indptr, adj.indices, w, feat)
+    for v in values:
+        if key == "spmm.scalar_path":
+            _lib.config_set("spmm.lpr", 64)
+        _lib.config_set(key, v)
+        assert np.array_equal(_run_mh(adj, feat, w), want), "%s=%d" % (key, v)

@@ -1,0 +1,264 @@
+"""Pins the CPU checker (oracle/) before anything is compared with it.
+
+Every check here is independent of the oracle's own formula text: library
+routines (scipy's csr.dot, numpy gather-sum, einsum: the closed forms the
+reference's own tests use, tests/test_module_spmm.py:29-30 and
+tests/test_module_sddmm.py:34-37), integer cases that float32 represents
+exactly, hand-computed cases where a different summation order or a fused
+multiply-add gives a different float, and structural invariants.
+"""
+import numpy as np
+import pytest
+import scipy.sparse
+
+from conftest import reference_test_matrix
+from featgraph_amd import datasets
+from featgraph_amd.util import util_convert_csr_to_dds
+from oracle import ref
+
+
+def _int_case(seed=0, shape=(61, 83), density=0.2, F=24):
+    """Small integers only: every product and partial sum is exact in float32."""
+    rng = np.random.default_rng(seed)
+    adj = scipy.sparse.random(shape[0], shape[1], density=density, format="csr", random_state=rng)
+    adj.data = rng.integers(1, 5, adj.nnz).astype(np.float32)
+    feat = rng.integers(-8, 9, (shape[1], F)).astype(np.float32)
+    return adj.astype(np.float32), feat
+
+
+# ---------------------------------------------------------------- SpMM (CSR, x86 nest)
+@pytest.mark.parametrize("P", [1, 4])
+def test_spmm_matches_scipy_like_the_reference_tests(adj_127x255, P):
+    adj = adj_127x255
+    feat = np.random.default_rng(1).random((adj.shape[1], 128), dtype=np.float32)
+    out = ref.spmm_csr_x86(adj.indptr, adj.indices, adj.data, feat, P)
+    np.testing.assert_allclose(adj.dot(feat), out, rtol=1e-4, atol=1e-4)  # the reference's own tolerance
+    exact = adj.astype(np.float64).dot(feat.astype(np.float64))
+    np.testing.assert_allclose(out, exact, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("P", [1, 2, 8])
+def test_spmm_exact_on_integers(P):
+    adj, feat = _int_case()
+    want = adj.astype(np.int64).dot(feat.astype(np.int64))
+    got = ref.spmm_csr_x86(adj.indptr, adj.indices, adj.data, feat, P)
+    assert np.array_equal(got, want.astype(np.float32))
+
+
+def test_spmm_nonsquare_shapes_and_empty_rows():
+    indptr = np.array([0, 0, 2, 2, 3], dtype=np.int32)      # rows 0 and 2 are empty
+    indices = np.array([4, 0, 2], dtype=np.int32)
+    vals = np.array([0.5, 2.0, 3.0], dtype=np.float32)
+    feat = np.arange(10, dtype=np.float32).reshape(5, 2) + 1
+    out = ref.spmm_csr_x86(indptr, indices, vals, feat)
+    want = np.array([[0, 0], [0.5 * 9 + 2 * 1, 0.5 * 10 + 2 * 2], [0, 0], [15, 18]], dtype=np.float32)
+    assert np.array_equal(out, want)
+    assert not np.signbit(out[0]).any()                       # empty rows are +0
+
+
+def test_spmm_sums_sequentially_in_csr_order():
+    # (((0 + 1e8) + 1) - 1e8) + 1 = 1 in float32; pairwise or reversed orders give 0 or 2
+    indptr = np.array([0, 4, 8], dtype=np.int32)
+    indices = np.array([0, 1, 2, 3, 3, 2, 1, 0], dtype=np.int32)
+    vals = np.ones(8, dtype=np.float32)
+    feat = np.array([[1e8], [1.0], [-1e8], [1.0]], dtype=np.float32)
+    out = ref.spmm_csr_x86(indptr, indices, vals, feat)
+    assert out[0, 0] == 1.0       # 1e8, 1, -1e8, 1
+    assert out[1, 0] == 0.0       # 1, -1e8, 1, 1e8 : ((1 - 1e8) + 1) + 1e8 = 0
+
+
+def test_spmm_rounds_product_and_sum_separately():
+    # v*x = 1 + 2^-11 + 2^-24 rounds to 1 + 2^-11; a fused multiply-add would leave 2^-24
+    v = np.float32(1 + 2.0 ** -12)
+    indptr = np.array([0, 2], dtype=np.int32)
+    indices = np.array([0, 1], dtype=np.int32)
+    vals = np.array([1.0, v], dtype=np.float32)
+    feat = np.array([[-(1 + 2.0 ** -11)], [v]], dtype=np.float32)
+    out = ref.spmm_csr_x86(indptr, indices, vals, feat)
+    assert out[0, 0] == 0.0
+
+
+def test_spmm_single_term_is_one_rounded_product():
+    rng = np.random.default_rng(3)
+    n = 50
+    indptr = np.arange(n + 1, dtype=np.int32)
+    indices = rng.integers(0, n, n).astype(np.int32)
+    vals = rng.random(n, dtype=np.float32)
+    feat = rng.standard_normal((n, 16), dtype=np.float32)
+    out = ref.spmm_csr_x86(indptr, indices, vals, feat)
+    assert np.array_equal(out, vals[:, None] * feat[indices])
+
+
+def test_spmm_tiling_and_row_permutation_do_not_change_bits(adj_127x255):
+    adj = adj_127x255
+    feat = np.random.default_rng(2).standard_normal((adj.shape[1], 64), dtype=np.float32)
+    base = ref.spmm_csr_x86(adj.indptr, adj.indices, adj.data, feat, 1)
+    for P in (2, 4, 16, 64):
+        assert np.array_equal(base, ref.spmm_csr_x86(adj.indptr, adj.indices, adj.data, feat, P))
+    perm = np.random.default_rng(5).permutation(adj.shape[0])
+    padj = adj[perm]
+    assert np.array_equal(base[perm], ref.spmm_csr_x86(padj.indptr, padj.indices, padj.data, feat, 1))
+
+
+def test_spmm_duplicate_and_unsorted_columns_add_in_stored_order():
+    indptr = np.array([0, 4], dtype=np.int32)
+    indices = np.array([2, 0, 2, 1], dtype=np.int32)
+    vals = np.array([1, 2, 3, 4], dtype=np.float32)
+    feat = np.array([[1.0], [10.0], [100.0]], dtype=np.float32)
+    assert ref.spmm_csr_x86(indptr, indices, vals, feat)[0, 0] == 100 + 2 + 300 + 40
+
+
+def test_spmm_linearity_on_integers():
+    adj, feat = _int_case(seed=4)
+    feat2 = np.random.default_rng(9).integers(-8, 9, feat.shape).astype(np.float32)
+    f = lambda x: ref.spmm_csr_x86(adj.indptr, adj.indices, adj.data, x)
+    assert np.array_equal(f(feat + feat2), f(feat) + f(feat2))
+
+
+def test_spmm_f64_matches_numpy_double(adj_127x255):
+    adj = adj_127x255
+    feat = np.random.default_rng(6).standard_normal((adj.shape[1], 33), dtype=np.float32)
+    want = adj.astype(np.float64).dot(feat.astype(np.float64))
+    np.testing.assert_allclose(ref.spmm_csr_f64(adj.indptr, adj.indices, adj.data, feat), want, rtol=1e-13, atol=1e-13)
+
+
+def test_spmm_rejects_indivisible_feature_tiling():
+    adj, feat = _int_case()
+    with pytest.raises(RuntimeError):
+        ref.spmm_csr_x86(adj.indptr, adj.indices, adj.data, feat, 5)
+
+
+# ---------------------------------------------------------------- SpMM (DDS, x86 nest)
+@pytest.mark.parametrize("P_col,P_feat", [(4, 1), (4, 4), (7, 2)])
+def test_dds_spmm_matches_scipy(adj_127x255, P_col, P_feat):
+    adj = adj_127x255
+    feat = np.random.default_rng(1).random((adj.shape[1], 128), dtype=np.float32)
+    s1_pos, s1_idx, vals = util_convert_csr_to_dds(adj, P_col)
+    out = ref.spmm_dds_x86(s1_pos, s1_idx, vals, feat, adj.shape[0], P_col, P_feat)
+    np.testing.assert_allclose(adj.dot(feat), out, rtol=1e-4, atol=1e-4)
+
+
+def test_dds_spmm_exact_on_integers_and_single_block_equals_csr():
+    adj, feat = _int_case(seed=7)
+    want = adj.astype(np.int64).dot(feat.astype(np.int64)).astype(np.float32)
+    for P_col in (1, 2, 5):
+        s1_pos, s1_idx, vals = util_convert_csr_to_dds(adj, P_col)
+        assert np.array_equal(ref.spmm_dds_x86(s1_pos, s1_idx, vals, feat, adj.shape[0], P_col, 2), want)
+    adj2 = reference_test_matrix("csr", seed=8)
+    feat2 = np.random.default_rng(8).standard_normal((adj2.shape[1], 32), dtype=np.float32)
+    s1_pos, s1_idx, vals = util_convert_csr_to_dds(adj2, 1)
+    assert np.array_equal(ref.spmm_dds_x86(s1_pos, s1_idx, vals, feat2, adj2.shape[0], 1, 1),
+                          ref.spmm_csr_x86(adj2.indptr, adj2.indices, adj2.data, feat2, 1))
+
+
+# ---------------------------------------------------------------- SDDMM
+def _closed_form_sddmm(coo, src, dst):
+    return (src[coo.col].astype(np.float64) * dst[coo.row].astype(np.float64)).sum(axis=-1)
+
+
+@pytest.mark.parametrize("P", [1, 4])
+def test_sddmm_matches_numpy_like_the_reference_tests(P):
+    coo = reference_test_matrix("coo", seed=0)
+    rng = np.random.default_rng(1)
+    src = rng.random((coo.shape[1], 128), dtype=np.float32)   # one row per COLUMN
+    dst = rng.random((coo.shape[0], 128), dtype=np.float32)   # one row per ROW
+    out = ref.sddmm_x86(coo.row, coo.col, src, dst, P)
+    np.testing.assert_allclose((src[coo.col] * dst[coo.row]).sum(axis=-1), out, rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(out, _closed_form_sddmm(coo, src, dst), rtol=1e-5, atol=1e-5)
+
+
+def test_sddmm_exact_on_integers_and_tiling_bits():
+    coo = reference_test_matrix("coo", seed=2, shape=(40, 70), density=0.3)
+    rng = np.random.default_rng(2)
+    src = rng.integers(-8, 9, (70, 24)).astype(np.float32)
+    dst = rng.integers(-8, 9, (40, 24)).astype(np.float32)
+    want = (src[coo.col].astype(np.int64) * dst[coo.row].astype(np.int64)).sum(-1).astype(np.float32)
+    for P in (1, 2, 3, 24):
+        assert np.array_equal(ref.sddmm_x86(coo.row, coo.col, src, dst, P), want)
+    srcf = rng.standard_normal((70, 24), dtype=np.float32)
+    dstf = rng.standard_normal((40, 24), dtype=np.float32)
+    base = ref.sddmm_x86(coo.row, coo.col, srcf, dstf, 1)
+    for P in (2, 4, 12):
+        assert np.array_equal(base, ref.sddmm_x86(coo.row, coo.col, srcf, dstf, P))
+
+
+def test_sddmm_src_goes_with_col_and_dst_with_row():
+    row = np.array([0, 1], dtype=np.int32)
+    col = np.array([2, 0], dtype=np.int32)
+    src = np.array([[1, 0], [0, 0], [0, 3]], dtype=np.float32)    # 3 columns
+    dst = np.array([[5, 7], [11, 13]], dtype=np.float32)          # 2 rows
+    out = ref.sddmm_x86(row, col, src, dst)
+    assert np.array_equal(out, np.array([3 * 7, 1 * 11], dtype=np.float32))
+
+
+def test_sddmm_sums_sequentially_in_k():
+    row = np.zeros(1, dtype=np.int32)
+    col = np.zeros(1, dtype=np.int32)
+    src = np.array([[1e8, 1.0, -1e8, 1.0]], dtype=np.float32)
+    dst = np.ones((1, 4), dtype=np.float32)
+    assert ref.sddmm_x86(row, col, src, dst)[0] == 1.0
+    assert ref.sddmm_x86(row, col, src, dst, 2)[0] == 1.0
+
+
+def test_sddmm_symmetry_permutation_duplicates():
+    coo = reference_test_matrix("coo", seed=3, shape=(30, 50), density=0.3)
+    rng = np.random.default_rng(3)
+    src = rng.standard_normal((50, 16), dtype=np.float32)
+    dst = rng.standard_normal((30, 16), dtype=np.float32)
+    base = ref.sddmm_x86(coo.row, coo.col, src, dst)
+    # swapping the roles on the transposed matrix gives the same products (multiplication commutes)
+    assert np.array_equal(base, ref.sddmm_x86(coo.col, coo.row, dst, src))
+    perm = rng.permutation(coo.nnz)
+    assert np.array_equal(base[perm], ref.sddmm_x86(coo.row[perm], coo.col[perm], src, dst))
+    row2, col2 = np.concatenate([coo.row, coo.row]), np.concatenate([coo.col, coo.col])
+    assert np.array_equal(np.concatenate([base, base]), ref.sddmm_x86(row2, col2, src, dst))
+
+
+def test_sddmm_fast_and_f64_variants_agree_with_closed_form():
+    coo = reference_test_matrix("coo", seed=4)
+    rng = np.random.default_rng(4)
+    src = rng.standard_normal((coo.shape[1], 100), dtype=np.float32)
+    dst = rng.standard_normal((coo.shape[0], 100), dtype=np.float32)
+    exact = _closed_form_sddmm(coo, src, dst)
+    np.testing.assert_allclose(ref.sddmm_f64(coo.row, coo.col, src, dst), exact, rtol=1e-13, atol=1e-13)
+    for par in (False, True):
+        np.testing.assert_allclose(ref.sddmm_x86_fast(coo.row, coo.col, src, dst, par), exact, rtol=1e-5, atol=1e-4)
+
+
+# ---------------------------------------------------------------- multi-head closed forms
+def test_sddmm_mh_matches_einsum_and_reduces_to_vanilla():
+    coo = reference_test_matrix("coo", seed=5, shape=(60, 45), density=0.2)
+    rng = np.random.default_rng(5)
+    src = rng.standard_normal((45, 8, 16), dtype=np.float32)
+    dst = rng.standard_normal((60, 8, 16), dtype=np.float32)
+    out = ref.sddmm_mh(coo.row, coo.col, src, dst)
+    want = np.einsum("ehd,ehd->eh", src[coo.col].astype(np.float64), dst[coo.row].astype(np.float64))
+    np.testing.assert_allclose(out, want, rtol=1e-5, atol=1e-5)
+    for h in range(8):   # head h alone is a vanilla SDDMM, bit for bit
+        assert np.array_equal(out[:, h], ref.sddmm_x86(coo.row, coo.col, np.ascontiguousarray(src[:, h]),
+                                                       np.ascontiguousarray(dst[:, h])))
+    isrc = rng.integers(-4, 5, (45, 3, 5)).astype(np.float32)
+    idst = rng.integers(-4, 5, (60, 3, 5)).astype(np.float32)
+    iwant = np.einsum("ehd,ehd->eh", isrc[coo.col].astype(np.int64), idst[coo.row].astype(np.int64))
+    assert np.array_equal(ref.sddmm_mh(coo.row, coo.col, isrc, idst), iwant.astype(np.float32))
+
+
+def test_spmm_mh_matches_per_head_scipy_and_reduces_to_vanilla():
+    adj = reference_test_matrix("csr", seed=6, shape=(70, 55), density=0.15)
+    rng = np.random.default_rng(6)
+    H, D = 4, 12
+    w = rng.random((adj.nnz, H), dtype=np.float32)
+    src = rng.standard_normal((55, H, D), dtype=np.float32)
+    out = ref.spmm_mh(adj.indptr, adj.indices, w, src)
+    for h in range(H):
+        a_h = scipy.sparse.csr_matrix((w[:, h].astype(np.float64), adj.indices, adj.indptr), shape=adj.shape)
+        np.testing.assert_allclose(out[:, h], a_h.dot(src[:, h].astype(np.float64)), rtol=1e-5, atol=1e-5)
+        assert np.array_equal(out[:, h], ref.spmm_csr_x86(adj.indptr, adj.indices, np.ascontiguousarray(w[:, h]),
+                                                          np.ascontiguousarray(src[:, h])))
+
+
+def test_softmax_weights_sum_to_one_per_row_and_head():
+    adj = datasets.config_graph("c4-mini")
+    w = datasets.softmax_edge_weights(adj, 8)
+    sums = np.add.reduceat(w.astype(np.float64), adj.indptr[:-1][np.diff(adj.indptr) > 0], axis=0)
+    np.testing.assert_allclose(sums, 1.0, rtol=0, atol=1e-5)
