@@ -126,15 +126,22 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_slot_kernel(const SpmmArgs
 #pragma unroll
       for (int u = 0; u < U; ++u) axpy(acc, v[u], x[u]);
     }
-    for (; j < n; ++j) {
-      const int c = slot_read<LPR>(my_col, j, lane);
-      const V x = fok ? *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F) : vzero<VEC>();
-      float v;
-      if (MH)
-        v = wp[static_cast<int64_t>(e + j) * a.H];
-      else
-        v = __int_as_float(slot_read<LPR>(__float_as_int(my_val), j, lane));
-      axpy(acc, v, x);
+    if (j < n) {  // fewer than U left: one masked batch, so these gathers overlap too
+      V x[U];
+      float v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int c = slot_read<LPR>(my_col, (j + u) & (LPR - 1), lane);
+        const bool live = j + u < n;
+        x[u] = (fok && live) ? *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F) : vzero<VEC>();
+        if (MH)
+          v[u] = live ? wp[static_cast<int64_t>(e + j + u) * a.H] : 0.0f;
+        else
+          v[u] = __int_as_float(slot_read<LPR>(__float_as_int(my_val), (j + u) & (LPR - 1), lane));
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (j + u < n) axpy(acc, v[u], x[u]);
     }
   }
   if (fok) *reinterpret_cast<V *>(a.out + static_cast<int64_t>(row) * F + f0) = acc;
@@ -187,15 +194,22 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_wave_kernel(const SpmmArgs
 #pragma unroll
       for (int u = 0; u < U; ++u) axpy(acc, v[u], x[u]);
     }
-    for (; j < n; ++j) {
-      const int c = __builtin_amdgcn_readlane(my_col, j);
-      const V x = fok ? *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F) : vzero<VEC>();
-      float v;
-      if (MH)
-        v = wp[static_cast<int64_t>(e + j) * a.H];
-      else
-        v = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_val), j));
-      axpy(acc, v, x);
+    if (j < n) {  // fewer than U left: one masked batch, so these gathers overlap too
+      V x[U];
+      float v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const bool live = j + u < n;  // wave-uniform
+        const int c = __builtin_amdgcn_readlane(my_col, (j + u) & (kWaveSize - 1));
+        x[u] = (fok && live) ? *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F) : vzero<VEC>();
+        if (MH)
+          v[u] = live ? wp[static_cast<int64_t>(e + j + u) * a.H] : 0.0f;
+        else
+          v[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_val), (j + u) & (kWaveSize - 1)));
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (j + u < n) axpy(acc, v[u], x[u]);
     }
   }
   if (fok) *reinterpret_cast<V *>(a.out + static_cast<int64_t>(row) * F + f0) = acc;
@@ -234,15 +248,19 @@ int dispatch_unroll(const SpmmArgs &a, const SpmmShape &s, hipStream_t stream) {
       case 4: return launch_wave<VEC, 4>(a, stream);
       case 8: return launch_wave<VEC, 8>(a, stream);
       case 16: return launch_wave<VEC, 16>(a, stream);
+      case 32: return launch_wave<VEC, 32>(a, stream);
     }
   } else {
     switch (s.unroll) {
       case 4: return launch_slot<VEC, LPR, 4>(a, stream);
       case 8: return launch_slot<VEC, LPR, 8>(a, stream);
       case 16: return launch_slot<VEC, LPR, 16>(a, stream);
+      case 32:
+        if (LPR >= 32) return launch_slot<VEC, (LPR >= 32 ? LPR : 32), 32>(a, stream);
+        break;
     }
   }
-  return fail(FG_EINVAL, "spmm unroll %d is not one of 4, 8, 16", s.unroll);
+  return fail(FG_EINVAL, "spmm unroll %d is not one of 4, 8, 16, 32 (32 needs 32 or 64 lanes per slot)", s.unroll);
 }
 
 template <int VEC>
@@ -270,16 +288,21 @@ SpmmShape spmm_choose_shape(const SpmmArgs &a, int feat_tiles) {
   const Config &cfg = config();
   SpmmShape s;
   const int max_vec = spmm_max_vec(a);
-  s.vec = (cfg.spmm_vec > 0 && cfg.spmm_vec <= max_vec) ? cfg.spmm_vec : max_vec;
-  // tile width asked for: the whole row, or about F / feat_tiles floats
-  int want = a.F;
-  if (feat_tiles > 1) want = (a.F + feat_tiles - 1) / feat_tiles;
+  // Tile width asked for.  By default 64 floats (one 256-byte gather per
+  // neighbour and wave): on the 232,965-vertex benchmark graph narrow tiles beat
+  // wide ones at every feature length, because each tile's column band of the
+  // feature matrix is what has to stay cache-resident while it is gathered from.
+  int want = a.F < 64 ? a.F : 64;
+  if (feat_tiles >= 1) want = (a.F + feat_tiles - 1) / feat_tiles;
+  int vec = 1;
+  while (vec < max_vec && (want + vec - 1) / vec > kWaveSize) vec *= 2;
+  s.vec = (cfg.spmm_vec > 0 && cfg.spmm_vec <= max_vec) ? cfg.spmm_vec : vec;
   int lanes = pow2_ceil((want + s.vec - 1) / s.vec);
   if (lanes < 8) lanes = 8;
   if (lanes > kWaveSize) lanes = kWaveSize;
   s.lpr = cfg.spmm_lpr > 0 ? cfg.spmm_lpr : lanes;
-  s.unroll = cfg.spmm_unroll > 0 ? cfg.spmm_unroll : 8;
-  s.scalar_path = cfg.spmm_scalar_path >= 0 ? cfg.spmm_scalar_path : 0;
+  s.unroll = cfg.spmm_unroll > 0 ? cfg.spmm_unroll : (s.lpr == 32 ? 32 : (s.lpr >= 16 ? 16 : 8));
+  s.scalar_path = cfg.spmm_scalar_path >= 0 ? cfg.spmm_scalar_path : 1;
   if (s.lpr != kWaveSize) s.scalar_path = 0;
   return s;
 }

@@ -38,16 +38,17 @@ def small_uniform_csr(n=4096, deg_lo=8, deg_hi=24, seed=0):
     return scipy.sparse.csr_matrix((vals, indices, indptr), shape=(n, n))
 
 
-def _sorted_unique_keys(keys):
+def _sorted_unique_keys(keys, use_gpu=None):
     """Sort int64 keys and drop duplicates.
 
     Sorting is a function of the values only, so the device used cannot change
     the result; a GPU, when torch sees one, merely makes the 114.6M-key case
-    take a fraction of a second instead of tens of seconds.
+    take a fraction of a second instead of tens of seconds.  use_gpu=False
+    forces the numpy path.
     """
     try:
         import torch
-        if torch.cuda.is_available():
+        if use_gpu is not False and torch.cuda.is_available():
             t = torch.from_numpy(keys).cuda()
             t = torch.unique(t, sorted=True)
             out = t.cpu().numpy()
@@ -63,7 +64,7 @@ def _sorted_unique_keys(keys):
     return keys[keep]
 
 
-def powerlaw_csr(n, mean_deg, sigma, max_deg, seed=0, self_loops=True):
+def powerlaw_csr(n, mean_deg, sigma, max_deg, seed=0, self_loops=True, use_gpu=None):
     """Power-law (lognormal out-degree) graph with uniform random columns.
 
     Degrees are clip(round(lognormal(mu, sigma)), 1, max_deg) with mu chosen so
@@ -87,7 +88,7 @@ def powerlaw_csr(n, mean_deg, sigma, max_deg, seed=0, self_loops=True):
     rows *= n
     rows += cols
     del cols
-    keys = _sorted_unique_keys(rows)
+    keys = _sorted_unique_keys(rows, use_gpu)
     del rows
     r = keys // n
     indices = (keys - r * n).astype(np.int32)
