@@ -7,6 +7,8 @@
 #include <cstring>
 #include <new>
 #include <numeric>
+#include <string>
+#include <cstdlib>
 #include <vector>
 
 #include "common.hpp"
@@ -37,6 +39,14 @@ struct fg_spmm_plan {
   int32_t *row_order;      // owned, device: rows by descending degree
   int32_t max_degree;
   int device;
+  // Row bounds in visiting order, optionally cut into column blocks:
+  // seg[b * n_rows + i] is the position of the first nonzero of row row_order[i]
+  // whose column id is >= b * block_cols, so block b of that row is
+  // [seg[b][i], seg[b+1][i]) and the whole row is [seg[0][i], seg[n_blocks][i]).
+  // n_blocks > 1 only when every row's column ids ascend.
+  int32_t *seg;  // owned, device, (n_blocks + 1) * n_rows entries
+  int32_t n_blocks;
+  int32_t block_cols;
 };
 
 namespace {
@@ -49,6 +59,27 @@ __global__ void count_out_of_range_kernel(const int32_t *idx, int64_t n, int64_t
     bad += (v < 0 || v >= bound) ? 1u : 0u;
   }
   if (bad) atomicAdd(n_bad, bad);
+}
+
+// One wave per row: writes the bounds of every column block of row row_order[i]
+// at position i, and raises *unsorted when two neighbouring column ids descend.
+__global__ void build_segments_kernel(const int32_t *indptr, const int32_t *indices, const int32_t *row_order,
+                                      int32_t n_rows, int32_t block_cols, int32_t n_blocks, int32_t *seg,
+                                      int *unsorted) {
+  const int i = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (i >= n_rows) return;
+  const int row = row_order[i];
+  const int start = indptr[row], end = indptr[row + 1];
+  for (int e = start + lane; e <= end; e += 64) {  // e == end is the sentinel that closes the last blocks
+    int bk = n_blocks, bp = -1;
+    if (e < end) bk = min(max(indices[e] / block_cols, 0), n_blocks - 1);
+    if (e > start) {
+      bp = min(max(indices[e - 1] / block_cols, 0), n_blocks - 1);
+      if (e < end && indices[e - 1] > indices[e]) atomicOr(unsorted, 1);
+    }
+    for (int b = bp + 1; b <= bk; ++b) seg[static_cast<int64_t>(b) * n_rows + i] = e;
+  }
 }
 
 int check_heads(int32_t H, int32_t D) {
@@ -71,7 +102,12 @@ int spmm_prepare(const fg_spmm_plan *plan, const float *feat, const float *w, fl
   a->feat = feat;
   a->out = out;
   a->row_order = (fg::config().spmm_sorted == 0) ? nullptr : plan->row_order;
+  if (a->row_order && plan->seg) {  // whole rows, in visiting order
+    a->seg_lo = plan->seg;
+    a->seg_hi = plan->seg + static_cast<int64_t>(plan->n_blocks) * plan->n_rows;
+  }
   a->n_rows = static_cast<int32_t>(plan->n_rows);
+  a->n_cols = static_cast<int32_t>(plan->n_cols);
   a->F = H * D;
   a->H = H;
   a->D = D;
@@ -79,6 +115,15 @@ int spmm_prepare(const fg_spmm_plan *plan, const float *feat, const float *w, fl
   a->n_tiles = (a->F + s->tile_width() - 1) / s->tile_width();
   a->n_slots = static_cast<int64_t>(a->n_tiles) * a->n_rows;
   return FG_OK;
+}
+
+bool use_column_blocks(const fg_spmm_plan *plan, const fg::SpmmArgs &a, const fg::SpmmShape &s) {
+  if (!plan->seg || plan->n_blocks < 2 || !a.row_order || fg::config().spmm_blocked == 0) return false;
+  if (fg::config().spmm_blocked > 0) return true;
+  // worthwhile only while the whole gathered band does not fit an L2 anyway
+  const int64_t band_bytes = static_cast<int64_t>(plan->n_cols) * std::min<int64_t>(s.tile_width(), a.F) * 4;
+  if (a.F < 64) return false;  // short feature rows: the single pass is faster (measured at 32 floats)
+  return band_bytes > (int64_t{6} << 20);
 }
 
 int sddmm_prepare(int64_t nnz, const int32_t *row, const int32_t *col, const float *src, const float *dst,
@@ -100,6 +145,61 @@ int sddmm_prepare(int64_t nnz, const int32_t *row, const int32_t *col, const flo
   return FG_OK;
 }
 
+// Builds the plan's bounds table.  Column blocks (n_blocks > 1) pay off when
+// the band of the feature matrix that one block gathers from (block_cols rows
+// of one 64-float tile, 4 MB by default) is about one XCD's L2 while the whole
+// matrix does not, and when a row still has enough nonzeros per block to
+// amortise re-reading its partial sum; otherwise the table holds whole rows.
+int build_bounds(fg_spmm_plan *p) {
+  const fg::Config &cfg = fg::config();
+  if (p->n_rows == 0) return FG_OK;
+  int64_t block_cols = cfg.spmm_block_cols > 0 ? cfg.spmm_block_cols : 16384;
+  int64_t n_blocks = (p->n_cols + block_cols - 1) / block_cols;
+  const double per_segment =
+      n_blocks > 0 ? static_cast<double>(p->nnz) / (static_cast<double>(p->n_rows) * n_blocks) : 0.0;
+  if (cfg.spmm_blocked == 0 || n_blocks < 2 || (cfg.spmm_blocked < 0 && per_segment < 8.0)) n_blocks = 1;
+  int *flag = nullptr;
+  FG_HIP_TRY(hipMalloc(&flag, sizeof(int)));
+  for (;;) {
+    if (n_blocks == 1) block_cols = 0x7fffffff;
+    int32_t *seg = nullptr;
+    hipError_t err = hipMalloc(&seg, static_cast<size_t>(n_blocks + 1) * p->n_rows * sizeof(int32_t));
+    if (err == hipErrorOutOfMemory && n_blocks > 1) {  // no room for the blocks: whole rows only
+      (void)hipGetLastError();
+      n_blocks = 1;
+      continue;
+    }
+    int unsorted = 0;
+    if (err == hipSuccess) err = hipMemset(flag, 0, sizeof(int));
+    if (err == hipSuccess) {
+      const int rows_per_block = 4;
+      const unsigned grid = static_cast<unsigned>((p->n_rows + rows_per_block - 1) / rows_per_block);
+      build_segments_kernel<<<dim3(grid), dim3(64 * rows_per_block)>>>(
+          p->indptr, p->indices, p->row_order, static_cast<int32_t>(p->n_rows), static_cast<int32_t>(block_cols),
+          static_cast<int32_t>(n_blocks), seg, flag);
+      err = hipGetLastError();
+    }
+    if (err == hipSuccess) err = hipMemcpy(&unsorted, flag, sizeof(int), hipMemcpyDeviceToHost);
+    if (err != hipSuccess) {
+      if (seg) (void)hipFree(seg);
+      (void)hipFree(flag);
+      return fg::fail(err == hipErrorOutOfMemory ? FG_ENOMEM : FG_EHIP, "row bounds construction: %s",
+                      hipGetErrorString(err));
+    }
+    if (unsorted && n_blocks > 1) {  // blocks would reorder the sums of such rows
+      (void)hipFree(seg);
+      n_blocks = 1;
+      continue;
+    }
+    p->seg = seg;
+    p->n_blocks = static_cast<int32_t>(n_blocks);
+    p->block_cols = static_cast<int32_t>(block_cols);
+    break;
+  }
+  (void)hipFree(flag);
+  return FG_OK;
+}
+
 int *config_slot(const char *key) {
   fg::Config &c = fg::config();
   if (!key) return nullptr;
@@ -108,10 +208,36 @@ int *config_slot(const char *key) {
   if (!strcmp(key, "spmm.unroll")) return &c.spmm_unroll;
   if (!strcmp(key, "spmm.scalar_path")) return &c.spmm_scalar_path;
   if (!strcmp(key, "spmm.sorted")) return &c.spmm_sorted;
+  if (!strcmp(key, "spmm.blocked")) return &c.spmm_blocked;
+  if (!strcmp(key, "spmm.block_cols")) return &c.spmm_block_cols;
+  if (!strcmp(key, "spmm.pipeline")) return &c.spmm_pipeline;
+  if (!strcmp(key, "spmm.pipe_blocks")) return &c.spmm_pipe_blocks;
   if (!strcmp(key, "sddmm.group")) return &c.sddmm_group;
   if (!strcmp(key, "sddmm.batches")) return &c.sddmm_batches;
   return nullptr;
 }
+
+// FEATGRAPH_HIP_CONFIG="key=value,key=value" applies fg_config_set pairs when the
+// library is loaded (handy under a profiler, where nothing else can reach in).
+struct EnvConfig {
+  EnvConfig() {
+    const char *env = getenv("FEATGRAPH_HIP_CONFIG");
+    if (!env) return;
+    std::string text(env);
+    size_t pos = 0;
+    while (pos < text.size()) {
+      size_t stop = text.find(',', pos);
+      if (stop == std::string::npos) stop = text.size();
+      const std::string item = text.substr(pos, stop - pos);
+      const size_t eq = item.find('=');
+      if (eq != std::string::npos) {
+        if (fg_config_set(item.substr(0, eq).c_str(), atoi(item.c_str() + eq + 1)) != FG_OK)
+          fprintf(stderr, "libfeatgraph_hip: ignoring FEATGRAPH_HIP_CONFIG item '%s'\n", item.c_str());
+      }
+      pos = stop + 1;
+    }
+  }
+};
 
 }  // namespace
 
@@ -178,6 +304,13 @@ int fg_spmm_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32
     delete p;
     return fg::fail(err == hipErrorOutOfMemory ? FG_ENOMEM : FG_EHIP, "plan upload: %s", hipGetErrorString(err));
   }
+  p->seg = nullptr;
+  p->n_blocks = 0;
+  p->block_cols = 0;
+  if (int rc = build_bounds(p)) {
+    fg_spmm_plan_destroy(p);
+    return rc;
+  }
   *plan = p;
   return FG_OK;
 }
@@ -185,6 +318,7 @@ int fg_spmm_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32
 void fg_spmm_plan_destroy(fg_spmm_plan *plan) {
   if (!plan) return;
   if (plan->row_order) (void)hipFree(plan->row_order);
+  if (plan->seg) (void)hipFree(plan->seg);
   delete plan;
 }
 
@@ -206,7 +340,24 @@ int fg_spmm_csr_mh_f32(const fg_spmm_plan *plan, const float *feat, const float 
   fg::SpmmArgs a;
   fg::SpmmShape s;
   if (int rc = spmm_prepare(plan, feat, w, out, H, D, feat_tiles, &a, &s)) return rc;
-  return fg::spmm_launch(a, s, static_cast<hipStream_t>(stream));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (!use_column_blocks(plan, a, s)) return fg::spmm_launch(a, s, st);
+  // One launch per (feature tile, column block), blocks in ascending column
+  // order: launches on one stream run one after the other, so every row's sum
+  // still grows in CSR order, carried from block to block in `out`.
+  const int n_tiles = a.n_tiles;
+  a.n_tiles = 1;
+  a.n_slots = a.n_rows;
+  for (int tile = 0; tile < n_tiles; ++tile) {
+    a.tile_base = tile;
+    for (int b = 0; b < plan->n_blocks; ++b) {
+      a.seg_lo = plan->seg + static_cast<int64_t>(b) * plan->n_rows;
+      a.seg_hi = a.seg_lo + plan->n_rows;
+      a.accumulate = b > 0;
+      if (int rc = fg::spmm_launch(a, s, st)) return rc;
+    }
+  }
+  return FG_OK;
 }
 
 int fg_sddmm_coo_f32(int64_t nnz, const int32_t *row, const int32_t *col, const float *src, const float *dst,
@@ -248,7 +399,8 @@ int fg_check_indices(int64_t n, const int32_t *idx, int64_t bound, int64_t *n_ba
 int fg_config_set(const char *key, int32_t value) {
   int *slot = config_slot(key);
   if (!slot) return fg::fail(FG_EINVAL, "unknown configuration key '%s'", key ? key : "(null)");
-  const bool flag = slot == &fg::config().spmm_scalar_path || slot == &fg::config().spmm_sorted;
+  const bool flag = slot == &fg::config().spmm_scalar_path || slot == &fg::config().spmm_sorted ||
+                    slot == &fg::config().spmm_blocked || slot == &fg::config().spmm_pipeline;
   // flags: 0 / 1 are explicit, anything negative restores the default;
   // sizes: 0 restores the default
   *slot = flag ? (value < 0 ? -1 : (value != 0)) : std::max(value, 0);
@@ -270,13 +422,20 @@ int fg_spmm_describe(const fg_spmm_plan *plan, int32_t H, int32_t D, int32_t fea
   alignas(16) static float dummy[4];
   if (int rc = spmm_prepare(plan, dummy, dummy, dummy, H, D, feat_tiles, &a, &s)) return rc;
   const int rows_per_wave = fg::kWaveSize / s.lpr;
-  const int64_t waves = (a.n_slots + rows_per_wave - 1) / rows_per_wave;
+  const bool blocked = use_column_blocks(plan, a, s);
+  const int64_t slots = blocked ? a.n_rows : a.n_slots;
+  const int64_t waves = (slots + rows_per_wave - 1) / rows_per_wave;
+  char passes[96] = "1 launch";
+  if (blocked)
+    snprintf(passes, sizeof(passes), "%d launches (%d tiles x %d column blocks of %d)", a.n_tiles * plan->n_blocks,
+             a.n_tiles, plan->n_blocks, plan->block_cols);
   snprintf(buf, static_cast<size_t>(cap),
            "spmm_csr rows=%lld cols=%lld nnz=%lld max_degree=%d H=%d D=%d | kernel=%s floats/lane=%d "
-           "lanes/row-slot=%d tile=%d floats x %d tiles gathers-in-flight=%d rows=%s | grid=%lld blocks x %d threads",
+           "lanes/row-slot=%d tile=%d floats x %d tiles gathers-in-flight=%d rows=%s | %s, grid=%lld blocks x %d "
+           "threads each",
            (long long)plan->n_rows, (long long)plan->n_cols, (long long)plan->nnz, plan->max_degree, H, D,
-           s.scalar_path ? "wave-per-row(scalar ids)" : "row-slot", s.vec, s.lpr, s.tile_width(), a.n_tiles,
-           s.unroll, a.row_order ? "by-descending-degree" : "natural",
+           s.pipeline ? "wave-per-row(pipelined)" : (s.scalar_path ? "wave-per-row(scalar ids)" : "row-slot"), s.vec, s.lpr, s.tile_width(), a.n_tiles,
+           s.unroll, a.row_order ? "by-descending-degree" : "natural", passes,
            (long long)((waves + fg::kWavesPerBlock - 1) / fg::kWavesPerBlock), fg::kBlockThreads);
   return FG_OK;
 }
@@ -299,3 +458,7 @@ int fg_sddmm_describe(int64_t nnz, int32_t H, int32_t D, char *buf, int64_t cap)
 }
 
 }  // extern "C"
+
+namespace {
+const EnvConfig g_env_config;
+}  // namespace

@@ -21,6 +21,7 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 // Launch-shape overrides (0 = library default).
 struct Config {
   int spmm_vec = 0, spmm_lpr = 0, spmm_unroll = 0, spmm_scalar_path = -1, spmm_sorted = -1;
+  int spmm_blocked = -1, spmm_block_cols = 0, spmm_pipeline = -1, spmm_pipe_blocks = 0;
   int sddmm_group = 0, sddmm_batches = 0;
 };
 Config &config();
@@ -39,15 +40,26 @@ struct SpmmArgs {
   float *out;
   const int32_t *row_order;  // rows by descending degree, or null for natural order
   int32_t n_rows;
+  int32_t n_cols;
   int32_t F;  // floats per feature row (= H * D)
   int32_t H;
   int32_t D;
   int32_t n_tiles;
   int64_t n_slots;  // n_tiles * n_rows
+  // Column-blocked passes: this launch covers only the nonzeros
+  // [seg_lo[row], seg_hi[row]) of every row (one column block), for the tiles
+  // tile_base .. tile_base + n_tiles - 1, and when `accumulate` is set it
+  // continues the sums that an earlier pass left in `out`.
+  const int32_t *seg_lo = nullptr;
+  const int32_t *seg_hi = nullptr;
+  int32_t tile_base = 0;
+  int32_t accumulate = 0;
 };
 
 struct SpmmShape {
   int vec, lpr, unroll, scalar_path;
+  int pipeline = 0;       // wave-per-row kernel that keeps three rows in flight
+  int pipe_blocks = 0;    // its grid size (workgroups per feature tile)
   int tile_width() const { return vec * lpr; }
 };
 

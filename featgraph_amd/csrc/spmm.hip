@@ -93,15 +93,20 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_slot_kernel(const SpmmArgs
   const int tile = static_cast<int>(slot / a.n_rows);
   const int i = static_cast<int>(slot - static_cast<int64_t>(tile) * a.n_rows);
   const int row = a.row_order ? a.row_order[i] : i;
-  const int f0 = tile * TW + sl * VEC;
+  const int f0 = (a.tile_base + tile) * TW + sl * VEC;
   const bool fok = f0 < a.F;  // lanes past the end of a partial last tile only take part in the cross-lane reads
   const int head = (MH && fok) ? f0 / a.D : 0;
   const int64_t F = a.F;
   const float *fp = a.feat + f0;
   const float *wp = a.w + head;
-  int e = a.indptr[row];
-  const int end = a.indptr[row + 1];
+  int e = a.seg_lo ? a.seg_lo[i] : a.indptr[row];
+  const int end = a.seg_lo ? a.seg_hi[i] : a.indptr[row + 1];
   V acc = vzero<VEC>();
+  float *const op = a.out + static_cast<int64_t>(row) * F + f0;
+  if (a.accumulate) {
+    if (e >= end) return;  // nothing of this row in this column block: the carried sum stays as it is
+    if (fok) acc = *reinterpret_cast<const V *>(op);
+  }
   for (; e < end; e += LPR) {
     const int n = min(LPR, end - e);
     int my_col = 0;
@@ -144,7 +149,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_slot_kernel(const SpmmArgs
         if (j + u < n) axpy(acc, v[u], x[u]);
     }
   }
-  if (fok) *reinterpret_cast<V *>(a.out + static_cast<int64_t>(row) * F + f0) = acc;
+  if (fok) *reinterpret_cast<V *>(op) = acc;
 }
 
 // Wave-per-(row, tile) kernel (LPR = 64): the row bounds and each neighbour's
@@ -161,15 +166,20 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_wave_kernel(const SpmmArgs
   const int tile = __builtin_amdgcn_readfirstlane(static_cast<int>(slot / a.n_rows));
   const int i = __builtin_amdgcn_readfirstlane(static_cast<int>(slot - static_cast<int64_t>(tile) * a.n_rows));
   const int row = __builtin_amdgcn_readfirstlane(a.row_order ? a.row_order[i] : i);
-  const int f0 = tile * TW + lane * VEC;
+  const int f0 = (a.tile_base + tile) * TW + lane * VEC;
   const bool fok = f0 < a.F;
   const int head = (MH && fok) ? f0 / a.D : 0;
   const int64_t F = a.F;
   const float *fp = a.feat + f0;
   const float *wp = a.w + head;
-  int e = __builtin_amdgcn_readfirstlane(a.indptr[row]);
-  const int end = __builtin_amdgcn_readfirstlane(a.indptr[row + 1]);
+  int e = __builtin_amdgcn_readfirstlane(a.seg_lo ? a.seg_lo[i] : a.indptr[row]);
+  const int end = __builtin_amdgcn_readfirstlane(a.seg_lo ? a.seg_hi[i] : a.indptr[row + 1]);
   V acc = vzero<VEC>();
+  float *const op = a.out + static_cast<int64_t>(row) * F + f0;
+  if (a.accumulate) {
+    if (e >= end) return;  // nothing of this row in this column block: the carried sum stays as it is
+    if (fok) acc = *reinterpret_cast<const V *>(op);
+  }
   for (; e < end; e += kWaveSize) {
     const int n = min(kWaveSize, end - e);
     int my_col = 0;
@@ -212,7 +222,160 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_wave_kernel(const SpmmArgs
         if (j + u < n) axpy(acc, v[u], x[u]);
     }
   }
-  if (fok) *reinterpret_cast<V *>(a.out + static_cast<int64_t>(row) * F + f0) = acc;
+  if (fok) *reinterpret_cast<V *>(op) = acc;
+}
+
+
+// Gathers for the B nonzeros j .. j+B-1 of the current 64-id block (only the
+// first `live` of them exist), then the B dependent adds.  `between` runs after
+// the gathers are issued and before their results are used: loads issued there
+// stay in flight while the adds wait only for the (older) gathers.
+template <int VEC, int B, bool MH, typename Between>
+__device__ __forceinline__ void gather_batch(typename VecOf<VEC>::type &acc, const float *fp, int64_t F, bool fok,
+                                             int col_reg, float val_reg, const float *wp, int64_t w_stride,
+                                             int64_t e0, int j, int live, Between between) {
+  using V = typename VecOf<VEC>::type;
+  V x[B];
+  float v[B];
+#pragma unroll
+  for (int u = 0; u < B; ++u) {
+    const bool on = u < live;  // wave-uniform
+    const int c = __builtin_amdgcn_readlane(col_reg, (j + u) & (kWaveSize - 1));
+    x[u] = (fok && on) ? *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F) : vzero<VEC>();
+    if (MH)
+      v[u] = on ? wp[(e0 + j + u) * w_stride] : 0.0f;
+    else
+      v[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(val_reg), (j + u) & (kWaveSize - 1)));
+  }
+  between();
+#pragma unroll
+  for (int u = 0; u < B; ++u)
+    if (u < live) axpy(acc, v[u], x[u]);
+}
+
+// Pipelined wave-per-row kernel.  A wave walks the rows wave, wave + W,
+// wave + 2W, ... of the plan's row list (W = waves in the grid) and keeps three
+// rows in flight: while it gathers for row k it has already asked for the first
+// 64 column ids / values (and, in a column-blocked pass, the carried sum) of row
+// k+1 and for the bounds of row k+2.  Short rows and short column-block
+// segments therefore cost one memory round trip each instead of four in a row.
+// blockIdx.y selects the feature tile.  Summation order per output element is
+// unchanged: CSR order, one lane per element.
+template <int VEC, int U, bool MH>
+__global__ __launch_bounds__(kBlockThreads) void spmm_pipe_kernel(const SpmmArgs a) {
+  using V = typename VecOf<VEC>::type;
+  constexpr int TW = VEC * kWaveSize;
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int n_waves = gridDim.x * kWavesPerBlock;
+  const int n = a.n_rows;
+  int item = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)));
+  const int f0 = (a.tile_base + static_cast<int>(blockIdx.y)) * TW + lane * VEC;
+  const bool fok = f0 < a.F;
+  const int head = (MH && fok) ? f0 / a.D : 0;
+  const int64_t F = a.F;
+  const float *fp = a.feat + f0;
+  const float *wp = a.w + head;
+  const int64_t w_stride = a.H;
+  const bool carry = a.accumulate != 0;
+
+  auto bounds = [&](int it, int &lo, int &hi, int &row) {
+    lo = hi = row = 0;
+    if (it < n) {
+      lo = a.seg_lo[it];
+      hi = a.seg_hi[it];
+      row = a.row_order[it];
+    }
+  };
+  auto first_block = [&](int lo, int hi, int row, int &col, float &val, V &acc) {
+    col = 0;
+    val = 0.0f;
+    acc = vzero<VEC>();
+    if (lane < hi - lo) {
+      col = a.indices[lo + lane];
+      if (!MH) val = a.w[lo + lane];
+    }
+    if (carry && hi > lo && fok) acc = *reinterpret_cast<const V *>(a.out + static_cast<int64_t>(row) * F + f0);
+  };
+
+  int lo_a, hi_a, row_a, col_a, lo_b, hi_b, row_b;
+  float val_a;
+  V acc_a;
+  bounds(item, lo_a, hi_a, row_a);
+  first_block(lo_a, hi_a, row_a, col_a, val_a, acc_a);
+  bounds(item + n_waves, lo_b, hi_b, row_b);
+
+  while (item < n) {
+    int lo_c, hi_c, row_c, col_b = 0;
+    float val_b = 0.0f;
+    V acc_b = vzero<VEC>();
+    bounds(item + 2 * n_waves, lo_c, hi_c, row_c);
+    bool next_asked = false;
+    auto ask_next = [&]() {  // first ids / values / carried sum of the next row, once, behind this row's first gathers
+      if (!next_asked) first_block(lo_b, hi_b, row_b, col_b, val_b, acc_b);
+      next_asked = true;
+    };
+    auto nothing = []() {};
+
+    int e = lo_a;
+    while (e < hi_a) {
+      const int cnt = min(kWaveSize, hi_a - e);
+      int col_n = 0;
+      float val_n = 0.0f;
+      auto ask_more = [&]() {  // the row's next 64 ids / values, behind this block's first gathers
+        ask_next();
+        const int more = hi_a - (e + kWaveSize);
+        if (lane < more) {
+          col_n = a.indices[e + kWaveSize + lane];
+          if (!MH) val_n = a.w[e + kWaveSize + lane];
+        }
+      };
+      int j = 0;
+      bool asked = false;
+      for (; j + U <= cnt; j += U) {
+        if (!asked)
+          gather_batch<VEC, U, MH>(acc_a, fp, F, fok, col_a, val_a, wp, w_stride, e, j, U, ask_more);
+        else
+          gather_batch<VEC, U, MH>(acc_a, fp, F, fok, col_a, val_a, wp, w_stride, e, j, U, nothing);
+        asked = true;
+      }
+      const int left = cnt - j;
+      if (left > 0) {
+        if (left > 8 || U <= 8) {
+          if (!asked)
+            gather_batch<VEC, U, MH>(acc_a, fp, F, fok, col_a, val_a, wp, w_stride, e, j, left, ask_more);
+          else
+            gather_batch<VEC, U, MH>(acc_a, fp, F, fok, col_a, val_a, wp, w_stride, e, j, left, nothing);
+        } else if (left > 4) {
+          if (!asked)
+            gather_batch<VEC, 8, MH>(acc_a, fp, F, fok, col_a, val_a, wp, w_stride, e, j, left, ask_more);
+          else
+            gather_batch<VEC, 8, MH>(acc_a, fp, F, fok, col_a, val_a, wp, w_stride, e, j, left, nothing);
+        } else {
+          if (!asked)
+            gather_batch<VEC, 4, MH>(acc_a, fp, F, fok, col_a, val_a, wp, w_stride, e, j, left, ask_more);
+          else
+            gather_batch<VEC, 4, MH>(acc_a, fp, F, fok, col_a, val_a, wp, w_stride, e, j, left, nothing);
+        }
+      }
+      e += kWaveSize;
+      col_a = col_n;
+      val_a = val_n;
+    }
+    ask_next();  // rows without nonzeros here never reached a gather
+    if (fok && (hi_a > lo_a || !carry))
+      *reinterpret_cast<V *>(a.out + static_cast<int64_t>(row_a) * F + f0) = acc_a;
+
+    lo_a = lo_b;
+    hi_a = hi_b;
+    row_a = row_b;
+    col_a = col_b;
+    val_a = val_b;
+    acc_a = acc_b;
+    lo_b = lo_c;
+    hi_b = hi_c;
+    row_b = row_c;
+    item += n_waves;
+  }
 }
 
 template <int VEC, int LPR, int U>
@@ -241,9 +404,33 @@ int launch_wave(const SpmmArgs &a, hipStream_t stream) {
   return FG_OK;
 }
 
+template <int VEC, int U>
+int launch_pipe(const SpmmArgs &a, const SpmmShape &s, hipStream_t stream) {
+  if (!a.seg_lo || !a.row_order) return fail(FG_EINVAL, "the pipelined kernel needs the plan's row list and bounds");
+  // a fixed number of resident waves, each walking many rows
+  int64_t blocks = static_cast<int64_t>(s.pipe_blocks);
+  const int64_t needed = (static_cast<int64_t>(a.n_rows) + kWavesPerBlock - 1) / kWavesPerBlock;
+  if (blocks > needed) blocks = needed;
+  if (blocks < 1) blocks = 1;
+  const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(a.n_tiles));
+  if (a.H > 1)
+    spmm_pipe_kernel<VEC, U, true><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+  else
+    spmm_pipe_kernel<VEC, U, false><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+  FG_HIP_TRY(hipGetLastError());
+  return FG_OK;
+}
+
 template <int VEC, int LPR>
 int dispatch_unroll(const SpmmArgs &a, const SpmmShape &s, hipStream_t stream) {
-  if (LPR == kWaveSize && s.scalar_path) {
+  if (LPR == kWaveSize && s.pipeline) {
+    switch (s.unroll) {
+      case 4: return launch_pipe<VEC, 4>(a, s, stream);
+      case 8: return launch_pipe<VEC, 8>(a, s, stream);
+      case 16: return launch_pipe<VEC, 16>(a, s, stream);
+      case 32: return launch_pipe<VEC, 32>(a, s, stream);
+    }
+  } else if (LPR == kWaveSize && s.scalar_path) {
     switch (s.unroll) {
       case 4: return launch_wave<VEC, 4>(a, stream);
       case 8: return launch_wave<VEC, 8>(a, stream);
@@ -293,17 +480,27 @@ SpmmShape spmm_choose_shape(const SpmmArgs &a, int feat_tiles) {
   // wide ones at every feature length, because each tile's column band of the
   // feature matrix is what has to stay cache-resident while it is gathered from.
   int want = a.F < 64 ? a.F : 64;
+  // ... unless even a 64-float band of the feature matrix is far beyond the
+  // 256 MB Infinity Cache (the 2.45M-vertex multi-head graph: 627 MB): then
+  // every gather goes to HBM whatever the tiling, and wider tiles win by
+  // reading the index and weight streams fewer times.
+  if (static_cast<int64_t>(a.n_cols) * 256 > (int64_t{192} << 20)) want = a.F < 128 ? a.F : 128;
   if (feat_tiles >= 1) want = (a.F + feat_tiles - 1) / feat_tiles;
   int vec = 1;
   while (vec < max_vec && (want + vec - 1) / vec > kWaveSize) vec *= 2;
   s.vec = (cfg.spmm_vec > 0 && cfg.spmm_vec <= max_vec) ? cfg.spmm_vec : vec;
   int lanes = pow2_ceil((want + s.vec - 1) / s.vec);
   if (lanes < 8) lanes = 8;
+  // a wave per row with idle lanes (pipelined kernel) beats two rows per wave at 17..63 floats
+  if (lanes > 16 && feat_tiles < 1) lanes = kWaveSize;
   if (lanes > kWaveSize) lanes = kWaveSize;
   s.lpr = cfg.spmm_lpr > 0 ? cfg.spmm_lpr : lanes;
   s.unroll = cfg.spmm_unroll > 0 ? cfg.spmm_unroll : (s.lpr == 32 ? 32 : (s.lpr >= 16 ? 16 : 8));
   s.scalar_path = cfg.spmm_scalar_path >= 0 ? cfg.spmm_scalar_path : 1;
   if (s.lpr != kWaveSize) s.scalar_path = 0;
+  s.pipeline = cfg.spmm_pipeline >= 0 ? cfg.spmm_pipeline : 1;
+  if (s.lpr != kWaveSize || !a.seg_lo || !a.row_order) s.pipeline = 0;
+  s.pipe_blocks = cfg.spmm_pipe_blocks > 0 ? cfg.spmm_pipe_blocks : 16384;
   return s;
 }
 

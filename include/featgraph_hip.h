@@ -55,8 +55,12 @@ FG_API const char *fg_last_error(void);
  * in the reference only uploads the three CSR arrays.  Reads indptr once
  * (device to host), checks that it starts at 0, is non-decreasing and ends at
  * nnz, and stores on the device the row ids sorted by descending degree (ties
- * by ascending row id).  The plan BORROWS indptr and indices: both must stay
- * alive and unchanged until fg_spmm_plan_destroy.
+ * by ascending row id).  When the matrix is wide and dense enough for column
+ * blocking to pay off and every row's column ids ascend, it also stores, per
+ * block of 16384 columns, where that block starts inside every row (one device
+ * pass over indices; (n_cols/16384 + 2) * n_rows int32).  The plan BORROWS
+ * indptr and indices: both must stay alive and unchanged until
+ * fg_spmm_plan_destroy.
  */
 FG_API int fg_spmm_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr,
                         const int32_t *indices, fg_spmm_plan **plan);
@@ -120,9 +124,14 @@ FG_API int fg_check_indices(int64_t n, const int32_t *idx, int64_t bound, int64_
  * slot: 8, 16, 32, 64), "spmm.unroll" (gathers in flight per lane: 4, 8, 16),
  * "spmm.scalar_path" (0/1: wave-per-row variant that keeps column ids in
  * scalar registers), "spmm.sorted" (0/1: visit rows by descending degree or
- * in natural order), "sddmm.group" (lanes per dot product: 1..16),
+ * in natural order), "spmm.blocked" (0/1: never / always run SpMM as one pass
+ * per column block when the plan has blocks; read at plan creation and at
+ * launch), "spmm.block_cols" (columns per block, read at plan creation),
+ * "spmm.pipeline" (0/1: wave-per-row kernel that keeps three rows in flight),
+ * "spmm.pipe_blocks" (its grid size),
+ * "sddmm.group" (lanes per dot product: 1..16),
  * "sddmm.batches" (64-edge batches per wave).  Value 0 restores the default of
- * a size; for the two 0/1 flags a negative value does.
+ * a size; for the 0/1 flags a negative value does.
  * The spmm.* keys change the launch shape only; "sddmm.group" also changes the
  * shape of the summation tree, i.e. the last bits of an SDDMM result.
  */

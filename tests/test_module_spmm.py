@@ -35,9 +35,9 @@ def _oracle(adj, feat_np, P=1):
 @pytest.fixture
 def config_guard():
     yield
-    for key in ("spmm.vec", "spmm.lpr", "spmm.unroll"):
+    for key in ("spmm.vec", "spmm.lpr", "spmm.unroll", "spmm.block_cols", "spmm.pipe_blocks"):
         _lib.config_set(key, 0)
-    for key in ("spmm.scalar_path", "spmm.sorted"):
+    for key in ("spmm.scalar_path", "spmm.sorted", "spmm.blocked", "spmm.pipeline"):
         _lib.config_set(key, -1)
 
 
@@ -111,9 +111,50 @@ def test_scalar_path_variants(config_guard, vec, unroll):
     feat = datasets.spmm_operands(adj, 256)
     _lib.config_set("spmm.lpr", 64)
     _lib.config_set("spmm.scalar_path", 1)
+    _lib.config_set("spmm.pipeline", 0)
     _lib.config_set("spmm.vec", vec)
     _lib.config_set("spmm.unroll", unroll)
     assert np.array_equal(_run_spmm(adj, feat), _oracle(adj, feat))
+
+
+@pytest.mark.parametrize("vec", [1, 2, 4])
+@pytest.mark.parametrize("unroll", [4, 8, 16, 32])
+@pytest.mark.parametrize("pipe_blocks", [1, 7, 2048])
+def test_pipelined_kernel_variants(config_guard, vec, unroll, pipe_blocks):
+    _lib.config_set("spmm.lpr", 64)
+    _lib.config_set("spmm.pipeline", 1)
+    _lib.config_set("spmm.vec", vec)
+    _lib.config_set("spmm.unroll", unroll)
+    _lib.config_set("spmm.pipe_blocks", pipe_blocks)
+    for name, F in (("c2-mini", 200), ("c4-mini", 64), ("c1", 64)):
+        adj = datasets.config_graph(name)
+        feat = datasets.spmm_operands(adj, F)
+        module = VanillaSpMMhip(adj)
+        assert "pipelined" in module.lower_to_ir([placeholder(feat.shape)], {}, {})
+        module.build([placeholder(feat.shape)], {}, {})
+        assert np.array_equal(module.run([nd.array(feat, module.ctx)]).asnumpy(), _oracle(adj, feat)), name
+
+
+def test_pipelined_kernel_on_degenerate_rows(config_guard):
+    _lib.config_set("spmm.lpr", 64)
+    _lib.config_set("spmm.pipeline", 1)
+    rng = np.random.default_rng(21)
+    # rows of length 0, 1, 63, 64, 65, 129 and a long one, fewer rows than waves
+    lens = np.array([0, 1, 63, 0, 64, 65, 129, 0, 0, 1000, 2, 0], dtype=np.int64)
+    indptr = np.zeros(len(lens) + 1, dtype=np.int32)
+    np.cumsum(lens, out=indptr[1:])
+    indices = np.concatenate([np.sort(rng.integers(0, 500, l)) for l in lens]).astype(np.int32)
+    vals = rng.random(indptr[-1], dtype=np.float32)
+    adj = scipy.sparse.csr_matrix((vals, indices, indptr), shape=(len(lens), 500))
+    feat = rng.standard_normal((500, 70), dtype=np.float32)
+    for blocked, block_cols in ((0, 0), (1, 64)):
+        _lib.config_set("spmm.blocked", blocked)
+        _lib.config_set("spmm.block_cols", block_cols)
+        module = VanillaSpMMhip(adj)
+        module.build([placeholder(feat.shape)], {}, {})
+        module.out_tvm.tensor.fill_(9.0)
+        out = module.run([nd.array(feat, module.ctx)]).asnumpy()
+        assert np.array_equal(out, ref.spmm_csr_x86(indptr, indices, vals, feat))
 
 
 def test_summation_order_and_unfused_rounding_on_the_gpu():
@@ -218,6 +259,72 @@ def test_index_check_entry_point():
     assert n_bad.value == 2
 
 
+# ---------------------------------------------------------------- column-blocked passes
+@pytest.mark.parametrize("block_cols", [7, 100, 1500])
+@pytest.mark.parametrize("shape", [(4, 16, 0), (1, 64, 1), (1, 64, 0), (2, 32, 0), (1, 32, 0), (1, 64, 2), (2, 64, 2)])
+def test_column_blocked_passes_give_the_same_bits(config_guard, block_cols, shape):
+    adj = datasets.config_graph("c2-mini")
+    _lib.config_set("spmm.blocked", 1)
+    _lib.config_set("spmm.block_cols", block_cols)
+    vec, lpr, kind = shape                      # kind: 0 row-slot kernel, 1 scalar-id kernel, 2 pipelined kernel
+    _lib.config_set("spmm.vec", vec)
+    _lib.config_set("spmm.lpr", lpr)
+    _lib.config_set("spmm.scalar_path", int(kind == 1))
+    _lib.config_set("spmm.pipeline", int(kind == 2))
+    for F in (64, 200):
+        feat = datasets.spmm_operands(adj, F)
+        module = VanillaSpMMhip(adj)
+        text = module.lower_to_ir([placeholder(feat.shape)], {}, {})
+        assert "column blocks of %d" % block_cols in text and ("pipelined" in text) == (kind == 2)
+        module.build([placeholder(feat.shape)], {}, {})
+        module.out_tvm.tensor.fill_(3.0)      # stale contents must not leak into the carried sums
+        out = module.run([nd.array(feat, module.ctx)]).asnumpy()
+        assert np.array_equal(out, _oracle(adj, feat)), "F=%d" % F
+
+
+def test_column_blocks_with_empty_rows_and_blocks(config_guard):
+    _lib.config_set("spmm.blocked", 1)
+    _lib.config_set("spmm.block_cols", 4)
+    rng = np.random.default_rng(11)
+    indptr = np.array([0, 0, 3, 3, 4, 9, 9], dtype=np.int32)
+    indices = np.array([0, 1, 30, 17, 2, 3, 3, 20, 31], dtype=np.int32)      # ascending, with a duplicate
+    vals = rng.random(9, dtype=np.float32)
+    adj = scipy.sparse.csr_matrix((vals, indices, indptr), shape=(6, 32))
+    feat = rng.standard_normal((32, 24), dtype=np.float32)
+    module = VanillaSpMMhip(adj)
+    assert "column blocks" in module.lower_to_ir([placeholder(feat.shape)], {}, {})
+    module.build([placeholder(feat.shape)], {}, {})
+    module.out_tvm.tensor.fill_(5.0)
+    out = module.run([nd.array(feat, module.ctx)]).asnumpy()
+    assert np.array_equal(out, ref.spmm_csr_x86(indptr, indices, vals, feat))
+
+
+def test_unsorted_columns_fall_back_to_the_single_pass(config_guard):
+    _lib.config_set("spmm.blocked", 1)
+    _lib.config_set("spmm.block_cols", 8)
+    rng = np.random.default_rng(12)
+    n = 300
+    indptr = np.arange(0, 40 * n + 1, 40, dtype=np.int32)
+    indices = rng.integers(0, 64, 40 * n).astype(np.int32)                    # not sorted inside rows
+    adj = scipy.sparse.csr_matrix((rng.random(40 * n, dtype=np.float32), indices, indptr), shape=(n, 64))
+    feat = rng.standard_normal((64, 64), dtype=np.float32)
+    module = VanillaSpMMhip(adj)
+    assert "1 launch" in module.lower_to_ir([placeholder(feat.shape)], {}, {})
+    module.build([placeholder(feat.shape)], {}, {})
+    out = module.run([nd.array(feat, module.ctx)]).asnumpy()
+    assert np.array_equal(out, ref.spmm_csr_x86(indptr, indices, adj.data, feat))
+
+
+def test_multihead_column_blocked(config_guard):
+    _lib.config_set("spmm.blocked", 1)
+    _lib.config_set("spmm.block_cols", 999)
+    adj = datasets.config_graph("c4-mini")
+    H, D = 8, 16
+    feat = datasets.spmm_operands(adj, (H, D))
+    w = datasets.softmax_edge_weights(adj, H)
+    assert np.array_equal(_run_mh(adj, feat, w), ref.spmm_mh(adj.indptr, adj.indices, w, feat))
+
+
 # ---------------------------------------------------------------- multi-head
 def _run_mh(adj, feat, w, compute_args=None):
     module = MultiHeadSpMMhip(adj)
@@ -244,7 +351,8 @@ def test_multihead_spmm_with_one_head_is_the_vanilla_kernel(config_guard):
         assert np.array_equal(_run_mh(adj, feat, adj.data.reshape(-1, 1).copy())[:, 0], vanilla)
 
 
-@pytest.mark.parametrize("key,values", [("spmm.vec", [1, 2, 4]), ("spmm.lpr", [8, 32, 64]), ("spmm.scalar_path", [1])])
+@pytest.mark.parametrize("key,values", [("spmm.vec", [1, 2, 4]), ("spmm.lpr", [8, 32, 64]), ("spmm.scalar_path", [1]),
+                                        ("spmm.pipeline", [1])])
 def test_multihead_launch_shapes_give_the_same_bits(config_guard, key, values):
     adj = datasets.config_graph("c4-mini")
     H, D = 8, 32
@@ -252,7 +360,7 @@ def test_multihead_launch_shapes_give_the_same_bits(config_guard, key, values):
     w = datasets.softmax_edge_weights(adj, H)
     want = ref.spmm_mh(adj.indptr, adj.indices, w, feat)
     for v in values:
-        if key == "spmm.scalar_path":
+        if key in ("spmm.scalar_path", "spmm.pipeline"):
             _lib.config_set("spmm.lpr", 64)
         _lib.config_set(key, v)
         assert np.array_equal(_run_mh(adj, feat, w), want), "%s=%d" % (key, v)
