@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <vector>
+
 #include "../../include/featgraph_hip.h"
 
 namespace fg {
@@ -22,7 +24,8 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 struct Config {
   int spmm_vec = 0, spmm_lpr = 0, spmm_unroll = 0, spmm_scalar_path = -1, spmm_sorted = -1;
   int spmm_blocked = -1, spmm_block_cols = 0, spmm_pipeline = -1, spmm_pipe_blocks = 0;
-  int sddmm_group = 0, sddmm_batches = 0;
+  int spmm_sweep = -1, spmm_sweep_waves_per_cu = 0;
+  int sddmm_group = 0, sddmm_batches = 0, sddmm_blocked = -1, sddmm_block_cols = 0;
 };
 Config &config();
 
@@ -64,6 +67,28 @@ struct SpmmShape {
 };
 
 SpmmShape spmm_choose_shape(const SpmmArgs &a, int feat_tiles);
+
+// Per-wave block-major nonzero lists for the column-sweep kernel
+// (spmm_sweep.hip); device arrays, owned by the SpMM plan.
+struct SweepPlan {
+  int32_t generations = 0;    // launches needed to cover all rows
+  int32_t waves = 0;          // waves per launch, all resident at once
+  int32_t rows_per_wave = 0;  // R
+  int32_t *rows = nullptr;    // [generations * waves * R] row id or -1
+  int32_t *ptr = nullptr;     // [generations * waves + 1] list bounds
+  int32_t *col = nullptr;     // [nnz] column id of each list entry
+  int32_t *src = nullptr;     // [nnz] its position in the CSR arrays (for the value / weight)
+  uint8_t *lrow = nullptr;    // [nnz] which of the wave's R rows it belongs to
+  int64_t max_load = 0, mean_load = 0;  // nonzeros per wave
+};
+
+// indptr / order: host copies of the CSR row pointer and of the plan's row
+// list; seg: the plan's device bounds table with n_blocks >= 2 column blocks.
+// Leaves *sp empty (generations == 0) when the lists are not worth building.
+int sweep_build(const std::vector<int32_t> &indptr, const std::vector<int32_t> &order, const int32_t *seg,
+                int32_t n_blocks, const int32_t *indices, int64_t nnz, SweepPlan *sp);
+void sweep_free(SweepPlan *sp);
+int sweep_launch(const SweepPlan &sp, const SpmmArgs &a, int unroll, hipStream_t stream);
 int spmm_launch(const SpmmArgs &a, const SpmmShape &s, hipStream_t stream);
 
 // One launch of the edge-parallel SDDMM kernel over n_ve = nnz * H dot
@@ -87,6 +112,23 @@ struct SddmmShape {
 
 SddmmShape sddmm_choose_shape(const SddmmArgs &a);
 int sddmm_launch(const SddmmArgs &a, const SddmmShape &s, hipStream_t stream);
+
+// Edge list of a COO matrix re-ordered by column block (sddmm_blocked.hip);
+// device arrays owned by the SDDMM plan, all null when blocking is not used.
+struct SddmmBlocks {
+  int32_t *row_p = nullptr;  // [nnz] row ids in block-major order
+  int32_t *col_p = nullptr;  // [nnz] column ids in block-major order
+  int32_t *pos_p = nullptr;  // [nnz] position of each of these edges in the caller's list
+  int32_t n_blocks = 0;
+  int32_t block_cols = 0;
+};
+
+int sddmm_blocks_build(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,
+                       SddmmBlocks *out);
+void sddmm_blocks_free(SddmmBlocks *b);
+// src / dst 16-byte aligned, F a multiple of 4.
+int sddmm_blocked_launch(const SddmmBlocks &b, int64_t nnz, const float *src, const float *dst, float *out, int32_t F,
+                         hipStream_t stream);
 
 inline bool aligned_to(const void *p, uintptr_t bytes) { return (reinterpret_cast<uintptr_t>(p) & (bytes - 1)) == 0; }
 

@@ -51,8 +51,24 @@ class SDDMMbase:
         C.require_device()
         self._adj_row_dev = torch.from_numpy(row).to(self._ctx)  # one upload per module (module/sddmm.py:59-60)
         self._adj_col_dev = torch.from_numpy(col).to(self._ctx)
+        # the cache-blocking step that the reference's constructor runs as 2-D partitioning on the host
+        # (module/sddmm.py:45-49) is a column-block plan on the device here; outputs stay in edge order
+        self._plan = ctypes.c_void_p()
+        with torch.cuda.device(self._ctx):
+            _lib.check(_lib.lib().fg_sddmm_plan_create(
+                self._nnz, self._num_rows, self._num_cols, self._adj_row_dev.data_ptr(),
+                self._adj_col_dev.data_ptr(), ctypes.byref(self._plan)))
         self._built = False
         self.out_tvm = None
+
+    def __del__(self):
+        plan = getattr(self, "_plan", None)
+        if plan:
+            try:
+                _lib.lib().fg_sddmm_plan_destroy(plan)
+            except Exception:
+                pass
+            self._plan = None
 
     def _register(self):
         raise NotImplementedError("Please register target and ctx.")
@@ -101,14 +117,14 @@ class SDDMMbase:
         """Description of the launch (module/sddmm.py:94-113 returns TVM IR)."""
         _, H, D = self._parse_build(input_placeholders, compute_args, schedule_args)
         buf = ctypes.create_string_buffer(1024)
-        _lib.check(_lib.lib().fg_sddmm_describe(self._nnz, H, D, buf, len(buf)))
+        _lib.check(_lib.lib().fg_sddmm_plan_describe(self._plan, H, D, buf, len(buf)))
         return buf.value.decode()
 
     def _launch(self, tensors):
         src, dst = tensors
-        _lib.check(_lib.lib().fg_sddmm_coo_mh_f32(
-            self._nnz, self._adj_row_dev.data_ptr(), self._adj_col_dev.data_ptr(), src.data_ptr(), dst.data_ptr(),
-            self.out_tvm.tensor.data_ptr(), self._H, self._D, C.current_stream_handle(self._ctx)))
+        _lib.check(_lib.lib().fg_sddmm_coo_plan_f32(
+            self._plan, src.data_ptr(), dst.data_ptr(), self.out_tvm.tensor.data_ptr(), self._H, self._D,
+            C.current_stream_handle(self._ctx)))
 
     def _checked_inputs(self, input_ndarrays):
         if not self._built:

@@ -104,6 +104,32 @@ FG_API int fg_sddmm_coo_f32(int64_t nnz, const int32_t *row, const int32_t *col,
                      float *out, int32_t F, void *stream);
 
 /*
+ * Cache-blocking schedule for one COO edge list; takes the place that
+ * SDDMMbase.__init__ gives to 2-D graph partitioning (module/sddmm.py:45-49):
+ * when the matrix is wide and dense enough, stores the edge list re-ordered by
+ * blocks of 16384 columns (stable, so each block keeps the caller's order)
+ * together with every edge's original position: 12 bytes per edge of device
+ * memory, built with one device radix sort.  Results are always written in the
+ * caller's edge order; there is no edge_mapping to apply.  The plan BORROWS row
+ * and col, which must stay alive and unchanged until fg_sddmm_plan_destroy.
+ */
+typedef struct fg_sddmm_plan fg_sddmm_plan;
+FG_API int fg_sddmm_plan_create(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,
+                                fg_sddmm_plan **plan);
+FG_API void fg_sddmm_plan_destroy(fg_sddmm_plan *plan);
+
+/*
+ * fg_sddmm_coo_mh_f32 on the plan's edge list.  With H = 1, F a multiple of 4
+ * and 16-byte aligned operands a blocked plan runs one launch per 64-float
+ * feature tile over the re-ordered list (each tile adds its partial dot
+ * product to Out, the reference's feature tiling: op/vanilla_sddmm.py:49-60);
+ * otherwise this is the plain kernel.  Both agree within float32 rounding.
+ */
+FG_API int fg_sddmm_coo_plan_f32(const fg_sddmm_plan *plan, const float *src, const float *dst, float *out, int32_t H,
+                                 int32_t D, void *stream);
+FG_API int fg_sddmm_plan_describe(const fg_sddmm_plan *plan, int32_t H, int32_t D, char *buf, int64_t cap);
+
+/*
  * Multi-head SDDMM (no counterpart in the reference; the edge function of
  * op/vanilla_sddmm.py:47 per head): Out[e, h] = sum_d src[col[e], h, d] * dst[row[e], h, d].
  * src [n_cols, H, D], dst [n_rows, H, D], out [nnz, H].  H = 1 gives
@@ -129,6 +155,8 @@ FG_API int fg_check_indices(int64_t n, const int32_t *idx, int64_t bound, int64_
  * launch), "spmm.block_cols" (columns per block, read at plan creation),
  * "spmm.pipeline" (0/1: wave-per-row kernel that keeps three rows in flight),
  * "spmm.pipe_blocks" (its grid size),
+ * "sddmm.blocked" (0/1: never / always build and use column blocks, read at
+ * plan creation), "sddmm.block_cols" (columns per block, read at plan creation),
  * "sddmm.group" (lanes per dot product: 1..16),
  * "sddmm.batches" (64-edge batches per wave).  Value 0 restores the default of
  * a size; for the 0/1 flags a negative value does.

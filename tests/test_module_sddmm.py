@@ -30,6 +30,8 @@ def config_guard():
     yield
     _lib.config_set("sddmm.group", 0)
     _lib.config_set("sddmm.batches", 0)
+    _lib.config_set("sddmm.block_cols", 0)
+    _lib.config_set("sddmm.blocked", -1)
 
 
 # the reference's own test on its matrix family (tests/test_module_sddmm.py:44-70)
@@ -120,6 +122,61 @@ def test_group_sizes_agree_within_rounding(config_guard):
     for g in (1, 2, 4, 8, 16):
         _lib.config_set("sddmm.group", g)
         np.testing.assert_allclose(_run_sddmm(coo, src, dst), want, rtol=RTOL, atol=ATOL)
+
+
+# ---------------------------------------------------------------- column-blocked edge list
+@pytest.mark.parametrize("F", [4, 32, 64, 100, 128, 260, 512])
+def test_column_blocked_edge_list(config_guard, F):
+    adj = datasets.config_graph("c2-mini")
+    coo = adj.tocoo()
+    src, dst = datasets.sddmm_operands(coo, F)
+    want = ref.sddmm_x86(coo.row, coo.col, src, dst)
+    exact = ref.sddmm_f64(coo.row, coo.col, src, dst)
+    _lib.config_set("sddmm.blocked", 0)
+    plain = _run_sddmm(coo, src, dst)
+    outs = []
+    for block_cols in (64, 1000):
+        _lib.config_set("sddmm.blocked", 1)
+        _lib.config_set("sddmm.block_cols", block_cols)
+        module = VanillaSDDMMhip(coo)
+        text = module.lower_to_ir([placeholder(src.shape), placeholder(dst.shape)], {}, {})
+        assert "column blocks of %d" % block_cols in text
+        module.build([placeholder(src.shape), placeholder(dst.shape)], {}, {})
+        module.out_tvm.tensor.fill_(7.0)                             # stale contents must not leak into the sums
+        out = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
+        np.testing.assert_allclose(out, want, rtol=RTOL, atol=ATOL)
+        np.testing.assert_allclose(out, exact, rtol=RTOL, atol=ATOL)
+        outs.append(out)
+    assert np.array_equal(outs[0], outs[1])                          # the block size only changes the visiting order
+    if F <= 64:
+        assert np.array_equal(outs[0], plain)                        # one tile: same summation tree as the plain kernel
+
+
+def test_column_blocked_edge_list_keeps_the_callers_edge_order(config_guard):
+    _lib.config_set("sddmm.blocked", 1)
+    _lib.config_set("sddmm.block_cols", 500)
+    coo = datasets.config_graph("c2-mini").tocoo()
+    rng = np.random.default_rng(8)
+    src = rng.integers(-8, 9, (coo.shape[1], 128)).astype(np.float32)
+    dst = rng.integers(-8, 9, (coo.shape[0], 128)).astype(np.float32)
+    perm = rng.permutation(coo.nnz)                                   # not row-sorted, with a ragged tail
+    perm = perm[:coo.nnz - 37]
+    shuffled = scipy.sparse.coo_matrix((coo.data[perm], (coo.row[perm], coo.col[perm])), shape=coo.shape)
+    want = (src[shuffled.col].astype(np.int64) * dst[shuffled.row].astype(np.int64)).sum(-1).astype(np.float32)
+    assert np.array_equal(_run_sddmm(shuffled, src, dst), want)      # exact on integers, in the caller's order
+
+
+def test_column_blocked_falls_back_for_odd_lengths_and_heads(config_guard):
+    _lib.config_set("sddmm.blocked", 1)
+    _lib.config_set("sddmm.block_cols", 500)
+    coo = datasets.config_graph("c2-mini").tocoo()
+    src, dst = datasets.sddmm_operands(coo, 30)
+    module = VanillaSDDMMhip(coo)
+    assert "column blocks" not in module.lower_to_ir([placeholder(src.shape), placeholder(dst.shape)], {}, {})
+    np.testing.assert_allclose(_run_sddmm(coo, src, dst), ref.sddmm_x86(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
+    src, dst = datasets.sddmm_operands(coo, (4, 16))
+    out = _run_sddmm(coo, src, dst, cls=MultiHeadSDDMMhip)
+    np.testing.assert_allclose(out, ref.sddmm_mh(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
 
 
 def test_module_surface(adj_127x255):
