@@ -226,6 +226,7 @@ int *config_slot(const char *key) {
   if (!strcmp(key, "spmm.block_cols")) return &c.spmm_block_cols;
   if (!strcmp(key, "spmm.pipeline")) return &c.spmm_pipeline;
   if (!strcmp(key, "spmm.sweep")) return &c.spmm_sweep;
+  if (!strcmp(key, "spmm.buffer_loads")) return &c.spmm_buffer_loads;
   if (!strcmp(key, "spmm.sweep_waves_per_cu")) return &c.spmm_sweep_waves_per_cu;
   if (!strcmp(key, "spmm.pipe_blocks")) return &c.spmm_pipe_blocks;
   if (!strcmp(key, "sddmm.group")) return &c.sddmm_group;
@@ -485,7 +486,8 @@ int fg_config_set(const char *key, int32_t value) {
   if (!slot) return fg::fail(FG_EINVAL, "unknown configuration key '%s'", key ? key : "(null)");
   const bool flag = slot == &fg::config().spmm_scalar_path || slot == &fg::config().spmm_sorted ||
                     slot == &fg::config().spmm_blocked || slot == &fg::config().spmm_pipeline ||
-                    slot == &fg::config().spmm_sweep || slot == &fg::config().sddmm_blocked;
+                    slot == &fg::config().spmm_sweep || slot == &fg::config().sddmm_blocked ||
+                    slot == &fg::config().spmm_buffer_loads;
   // flags: 0 / 1 are explicit, anything negative restores the default;
   // sizes: 0 restores the default
   *slot = flag ? (value < 0 ? -1 : (value != 0)) : std::max(value, 0);

@@ -24,7 +24,7 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 struct Config {
   int spmm_vec = 0, spmm_lpr = 0, spmm_unroll = 0, spmm_scalar_path = -1, spmm_sorted = -1;
   int spmm_blocked = -1, spmm_block_cols = 0, spmm_pipeline = -1, spmm_pipe_blocks = 0;
-  int spmm_sweep = -1, spmm_sweep_waves_per_cu = 0;
+  int spmm_sweep = -1, spmm_sweep_waves_per_cu = 0, spmm_buffer_loads = -1;
   int sddmm_group = 0, sddmm_batches = 0, sddmm_blocked = -1, sddmm_block_cols = 0;
 };
 Config &config();

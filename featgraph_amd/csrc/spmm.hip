@@ -97,7 +97,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_slot_kernel(const SpmmArgs
   const bool fok = f0 < a.F;  // lanes past the end of a partial last tile only take part in the cross-lane reads
   const int head = (MH && fok) ? f0 / a.D : 0;
   const int64_t F = a.F;
-  const float *fp = a.feat + f0;
+  const float *fp = a.feat + (fok ? f0 : a.F - VEC);  // lanes past a partial tile re-read its last group and never store
   const float *wp = a.w + head;
   int e = a.seg_lo ? a.seg_lo[i] : a.indptr[row];
   const int end = a.seg_lo ? a.seg_hi[i] : a.indptr[row + 1];
@@ -122,7 +122,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_slot_kernel(const SpmmArgs
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int c = slot_read<LPR>(my_col, j + u, lane);
-        x[u] = fok ? *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F) : vzero<VEC>();
+        x[u] = *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F);
         if (MH)
           v[u] = wp[static_cast<int64_t>(e + j + u) * a.H];
         else
@@ -138,7 +138,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_slot_kernel(const SpmmArgs
       for (int u = 0; u < U; ++u) {
         const int c = slot_read<LPR>(my_col, (j + u) & (LPR - 1), lane);
         const bool live = j + u < n;
-        x[u] = (fok && live) ? *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F) : vzero<VEC>();
+        x[u] = live ? *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F) : vzero<VEC>();
         if (MH)
           v[u] = live ? wp[static_cast<int64_t>(e + j + u) * a.H] : 0.0f;
         else
@@ -170,7 +170,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_wave_kernel(const SpmmArgs
   const bool fok = f0 < a.F;
   const int head = (MH && fok) ? f0 / a.D : 0;
   const int64_t F = a.F;
-  const float *fp = a.feat + f0;
+  const float *fp = a.feat + (fok ? f0 : a.F - VEC);  // lanes past a partial tile re-read its last group and never store
   const float *wp = a.w + head;
   int e = __builtin_amdgcn_readfirstlane(a.seg_lo ? a.seg_lo[i] : a.indptr[row]);
   const int end = __builtin_amdgcn_readfirstlane(a.seg_lo ? a.seg_hi[i] : a.indptr[row + 1]);
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_wave_kernel(const SpmmArgs
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int c = __builtin_amdgcn_readlane(my_col, j + u);
-        x[u] = fok ? *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F) : vzero<VEC>();
+        x[u] = *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F);
         if (MH)
           v[u] = wp[static_cast<int64_t>(e + j + u) * a.H];
         else
@@ -211,7 +211,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_wave_kernel(const SpmmArgs
       for (int u = 0; u < U; ++u) {
         const bool live = j + u < n;  // wave-uniform
         const int c = __builtin_amdgcn_readlane(my_col, (j + u) & (kWaveSize - 1));
-        x[u] = (fok && live) ? *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F) : vzero<VEC>();
+        x[u] = live ? *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F) : vzero<VEC>();
         if (MH)
           v[u] = live ? wp[static_cast<int64_t>(e + j + u) * a.H] : 0.0f;
         else
@@ -226,12 +226,49 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_wave_kernel(const SpmmArgs
 }
 
 
-// Gathers for the B nonzeros j .. j+B-1 of the current 64-id block (only the
-// first `live` of them exist), then the B dependent adds.  `between` runs after
-// the gathers are issued and before their results are used: loads issued there
-// stay in flight while the adds wait only for the (older) gathers.
-template <int VEC, int B, bool MH, typename Between>
-__device__ __forceinline__ void gather_batch(typename VecOf<VEC>::type &acc, const float *fp, int64_t F, bool fok,
+// One neighbour row's VEC floats for this lane.  With BUF the feature matrix is
+// addressed as a buffer resource: the load takes the lane's fixed byte offset in
+// a vector register and the row's byte offset (column id * row bytes) in a
+// scalar register, so a gather costs one scalar multiply and no vector
+// arithmetic; it needs the whole matrix to span less than 4 GiB.  Otherwise the
+// address is formed per lane in 64 bits.  Lanes past the end of a partial
+// tile carry the offset of the row's last valid group and never store.
+template <int VEC, bool BUF>
+struct RowGather {
+  using V = typename VecOf<VEC>::type;
+  __amdgpu_buffer_rsrc_t rsrc;
+  const char *base;
+  int64_t row_bytes;
+  uint32_t lane_off;
+
+  __device__ __forceinline__ RowGather(const float *feat, int64_t n_rows, int64_t F, uint32_t lane_off_)
+      : base(reinterpret_cast<const char *>(feat)), row_bytes(F * 4), lane_off(lane_off_) {
+    // word 3 of the descriptor: 32-bit untyped data, as gfx9-family buffer loads expect
+    rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(feat), 0,
+                                             BUF ? static_cast<int>(static_cast<uint32_t>(n_rows * F * 4)) : 0,
+                                             0x00020000);
+  }
+  __device__ __forceinline__ V load(int col) const {  // col is wave-uniform
+    if constexpr (BUF) {
+      const int soff = col * static_cast<int>(row_bytes);
+      if constexpr (VEC == 1)
+        return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b32(rsrc, static_cast<int>(lane_off), soff, 0));
+      else if constexpr (VEC == 2)
+        return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b64(rsrc, static_cast<int>(lane_off), soff, 0));
+      else
+        return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b128(rsrc, static_cast<int>(lane_off), soff, 0));
+    } else {
+      return *reinterpret_cast<const V *>(base + static_cast<int64_t>(col) * row_bytes + lane_off);
+    }
+  }
+};
+
+// Gathers for the B nonzeros j .. j+B-1 of the current 64-id block (when !FULL
+// only the first `live` of them exist), then the B dependent adds.  `between`
+// runs after the gathers are issued and before their results are used: loads
+// issued there stay in flight while the adds wait only for the (older) gathers.
+template <int VEC, int B, bool MH, bool FULL, bool BUF, typename Between>
+__device__ __forceinline__ void gather_batch(typename VecOf<VEC>::type &acc, const RowGather<VEC, BUF> &feat,
                                              int col_reg, float val_reg, const float *wp, int64_t w_stride,
                                              int64_t e0, int j, int live, Between between) {
   using V = typename VecOf<VEC>::type;
@@ -239,9 +276,9 @@ __device__ __forceinline__ void gather_batch(typename VecOf<VEC>::type &acc, con
   float v[B];
 #pragma unroll
   for (int u = 0; u < B; ++u) {
-    const bool on = u < live;  // wave-uniform
+    const bool on = FULL || u < live;  // wave-uniform
     const int c = __builtin_amdgcn_readlane(col_reg, (j + u) & (kWaveSize - 1));
-    x[u] = (fok && on) ? *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F) : vzero<VEC>();
+    x[u] = on ? feat.load(c) : vzero<VEC>();
     if (MH)
       v[u] = on ? wp[(e0 + j + u) * w_stride] : 0.0f;
     else
@@ -250,7 +287,7 @@ __device__ __forceinline__ void gather_batch(typename VecOf<VEC>::type &acc, con
   between();
 #pragma unroll
   for (int u = 0; u < B; ++u)
-    if (u < live) axpy(acc, v[u], x[u]);
+    if (FULL || u < live) axpy(acc, v[u], x[u]);
 }
 
 // Pipelined wave-per-row kernel.  A wave walks the rows wave, wave + W,
@@ -261,7 +298,7 @@ __device__ __forceinline__ void gather_batch(typename VecOf<VEC>::type &acc, con
 // segments therefore cost one memory round trip each instead of four in a row.
 // blockIdx.y selects the feature tile.  Summation order per output element is
 // unchanged: CSR order, one lane per element.
-template <int VEC, int U, bool MH>
+template <int VEC, int U, bool MH, bool BUF>
 __global__ __launch_bounds__(kBlockThreads) void spmm_pipe_kernel(const SpmmArgs a) {
   using V = typename VecOf<VEC>::type;
   constexpr int TW = VEC * kWaveSize;
@@ -273,7 +310,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_pipe_kernel(const SpmmArgs
   const bool fok = f0 < a.F;
   const int head = (MH && fok) ? f0 / a.D : 0;
   const int64_t F = a.F;
-  const float *fp = a.feat + f0;
+  const RowGather<VEC, BUF> feat(a.feat, a.n_cols, F, static_cast<uint32_t>(fok ? f0 : a.F - VEC) * 4u);
   const float *wp = a.w + head;
   const int64_t w_stride = a.H;
   const bool carry = a.accumulate != 0;
@@ -333,28 +370,28 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_pipe_kernel(const SpmmArgs
       bool asked = false;
       for (; j + U <= cnt; j += U) {
         if (!asked)
-          gather_batch<VEC, U, MH>(acc_a, fp, F, fok, col_a, val_a, wp, w_stride, e, j, U, ask_more);
+          gather_batch<VEC, U, MH, true, BUF>(acc_a, feat, col_a, val_a, wp, w_stride, e, j, U, ask_more);
         else
-          gather_batch<VEC, U, MH>(acc_a, fp, F, fok, col_a, val_a, wp, w_stride, e, j, U, nothing);
+          gather_batch<VEC, U, MH, true, BUF>(acc_a, feat, col_a, val_a, wp, w_stride, e, j, U, nothing);
         asked = true;
       }
       const int left = cnt - j;
       if (left > 0) {
         if (left > 8 || U <= 8) {
           if (!asked)
-            gather_batch<VEC, U, MH>(acc_a, fp, F, fok, col_a, val_a, wp, w_stride, e, j, left, ask_more);
+            gather_batch<VEC, U, MH, false, BUF>(acc_a, feat, col_a, val_a, wp, w_stride, e, j, left, ask_more);
           else
-            gather_batch<VEC, U, MH>(acc_a, fp, F, fok, col_a, val_a, wp, w_stride, e, j, left, nothing);
+            gather_batch<VEC, U, MH, false, BUF>(acc_a, feat, col_a, val_a, wp, w_stride, e, j, left, nothing);
         } else if (left > 4) {
           if (!asked)
-            gather_batch<VEC, 8, MH>(acc_a, fp, F, fok, col_a, val_a, wp, w_stride, e, j, left, ask_more);
+            gather_batch<VEC, 8, MH, false, BUF>(acc_a, feat, col_a, val_a, wp, w_stride, e, j, left, ask_more);
           else
-            gather_batch<VEC, 8, MH>(acc_a, fp, F, fok, col_a, val_a, wp, w_stride, e, j, left, nothing);
+            gather_batch<VEC, 8, MH, false, BUF>(acc_a, feat, col_a, val_a, wp, w_stride, e, j, left, nothing);
         } else {
           if (!asked)
-            gather_batch<VEC, 4, MH>(acc_a, fp, F, fok, col_a, val_a, wp, w_stride, e, j, left, ask_more);
+            gather_batch<VEC, 4, MH, false, BUF>(acc_a, feat, col_a, val_a, wp, w_stride, e, j, left, ask_more);
           else
-            gather_batch<VEC, 4, MH>(acc_a, fp, F, fok, col_a, val_a, wp, w_stride, e, j, left, nothing);
+            gather_batch<VEC, 4, MH, false, BUF>(acc_a, feat, col_a, val_a, wp, w_stride, e, j, left, nothing);
         }
       }
       e += kWaveSize;
@@ -413,10 +450,19 @@ int launch_pipe(const SpmmArgs &a, const SpmmShape &s, hipStream_t stream) {
   if (blocks > needed) blocks = needed;
   if (blocks < 1) blocks = 1;
   const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(a.n_tiles));
-  if (a.H > 1)
-    spmm_pipe_kernel<VEC, U, true><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
-  else
-    spmm_pipe_kernel<VEC, U, false><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+  // buffer addressing needs the feature matrix to span less than 4 GiB
+  const bool buf = static_cast<int64_t>(a.n_cols) * a.F * 4 < (int64_t{1} << 32) && config().spmm_buffer_loads != 0;
+  if (a.H > 1) {
+    if (buf)
+      spmm_pipe_kernel<VEC, U, true, true><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+    else
+      spmm_pipe_kernel<VEC, U, true, false><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+  } else {
+    if (buf)
+      spmm_pipe_kernel<VEC, U, false, true><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+    else
+      spmm_pipe_kernel<VEC, U, false, false><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+  }
   FG_HIP_TRY(hipGetLastError());
   return FG_OK;
 }

@@ -154,7 +154,11 @@ FG_API int fg_check_indices(int64_t n, const int32_t *idx, int64_t bound, int64_
  * per column block when the plan has blocks; read at plan creation and at
  * launch), "spmm.block_cols" (columns per block, read at plan creation),
  * "spmm.pipeline" (0/1: wave-per-row kernel that keeps three rows in flight),
- * "spmm.pipe_blocks" (its grid size),
+ * "spmm.pipe_blocks" (its grid size), "spmm.buffer_loads" (0/1: gather through
+ * a buffer resource with scalar row offsets; needs a feature matrix below 4 GiB),
+ * "spmm.sweep" (1: also build, and use, the per-wave block-major lists of the
+ * experimental column-sweep kernel; read at plan creation and at launch),
+ * "spmm.sweep_waves_per_cu" (its resident waves per CU),
  * "sddmm.blocked" (0/1: never / always build and use column blocks, read at
  * plan creation), "sddmm.block_cols" (columns per block, read at plan creation),
  * "sddmm.group" (lanes per dot product: 1..16),

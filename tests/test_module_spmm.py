@@ -38,7 +38,8 @@ def config_guard():
     for key in ("spmm.vec", "spmm.lpr", "spmm.unroll", "spmm.block_cols", "spmm.pipe_blocks",
                 "spmm.sweep_waves_per_cu"):
         _lib.config_set(key, 0)
-    for key in ("spmm.scalar_path", "spmm.sorted", "spmm.blocked", "spmm.pipeline", "spmm.sweep"):
+    for key in ("spmm.scalar_path", "spmm.sorted", "spmm.blocked", "spmm.pipeline", "spmm.sweep",
+                "spmm.buffer_loads"):
         _lib.config_set(key, -1)
 
 
@@ -134,6 +135,17 @@ def test_pipelined_kernel_variants(config_guard, vec, unroll, pipe_blocks):
         assert "pipelined" in module.lower_to_ir([placeholder(feat.shape)], {}, {})
         module.build([placeholder(feat.shape)], {}, {})
         assert np.array_equal(module.run([nd.array(feat, module.ctx)]).asnumpy(), _oracle(adj, feat)), name
+
+
+def test_pipelined_kernel_without_buffer_addressing(config_guard):
+    _lib.config_set("spmm.lpr", 64)
+    _lib.config_set("spmm.pipeline", 1)
+    _lib.config_set("spmm.buffer_loads", 0)
+    for vec in (1, 4):
+        _lib.config_set("spmm.vec", vec)
+        adj = datasets.config_graph("c2-mini")
+        feat = datasets.spmm_operands(adj, 200)
+        assert np.array_equal(_run_spmm(adj, feat), _oracle(adj, feat))
 
 
 def test_pipelined_kernel_on_degenerate_rows(config_guard):
