@@ -140,8 +140,10 @@ bool use_column_blocks(const fg_spmm_plan *plan, const fg::SpmmArgs &a, const fg
   return band_bytes > (int64_t{6} << 20);
 }
 
+// n_rows / n_cols: matrix extents when known (a plan knows them), else 0.
 int sddmm_prepare(int64_t nnz, const int32_t *row, const int32_t *col, const float *src, const float *dst,
-                  float *out, int32_t H, int32_t D, fg::SddmmArgs *a, fg::SddmmShape *s) {
+                  float *out, int32_t H, int32_t D, fg::SddmmArgs *a, fg::SddmmShape *s, int64_t n_rows = 0,
+                  int64_t n_cols = 0) {
   if (nnz < 0) return fg::fail(FG_EINVAL, "nnz = %lld is negative", (long long)nnz);
   if (int rc = check_heads(H, D)) return rc;
   if (nnz > 0 && (!row || !col || !src || !dst || !out)) return fg::fail(FG_EINVAL, "a data pointer is null");
@@ -154,6 +156,8 @@ int sddmm_prepare(int64_t nnz, const int32_t *row, const int32_t *col, const flo
   a->H = H;
   a->D = D;
   a->stride = H * D;
+  if (n_rows > 0) a->dst_bytes = n_rows * H * D * 4;
+  if (n_cols > 0) a->src_bytes = n_cols * H * D * 4;
   *s = fg::sddmm_choose_shape(*a);
   a->batches = s->batches;
   return FG_OK;
@@ -233,6 +237,8 @@ int *config_slot(const char *key) {
   if (!strcmp(key, "sddmm.batches")) return &c.sddmm_batches;
   if (!strcmp(key, "sddmm.blocked")) return &c.sddmm_blocked;
   if (!strcmp(key, "sddmm.block_cols")) return &c.sddmm_block_cols;
+  if (!strcmp(key, "sddmm.fast")) return &c.sddmm_fast;
+  if (!strcmp(key, "sddmm.buffer_loads")) return &c.sddmm_buffer_loads;
   return nullptr;
 }
 
@@ -437,11 +443,17 @@ static bool sddmm_use_blocks(const fg_sddmm_plan *plan, const float *src, const 
 int fg_sddmm_coo_plan_f32(const fg_sddmm_plan *plan, const float *src, const float *dst, float *out, int32_t H,
                           int32_t D, void *stream) {
   if (!plan) return fg::fail(FG_EINVAL, "plan is null");
-  if (!sddmm_use_blocks(plan, src, dst, H, D))
-    return fg_sddmm_coo_mh_f32(plan->nnz, plan->row, plan->col, src, dst, out, H, D, stream);
+  if (!sddmm_use_blocks(plan, src, dst, H, D)) {
+    fg::SddmmArgs a;
+    fg::SddmmShape s;
+    if (int rc = sddmm_prepare(plan->nnz, plan->row, plan->col, src, dst, out, H, D, &a, &s, plan->n_rows, plan->n_cols))
+      return rc;
+    return fg::sddmm_launch(a, s, static_cast<hipStream_t>(stream));
+  }
   if (int rc = check_heads(H, D)) return rc;
   if (!src || !dst || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
-  return fg::sddmm_blocked_launch(plan->blocks, plan->nnz, src, dst, out, D, static_cast<hipStream_t>(stream));
+  return fg::sddmm_blocked_launch(plan->blocks, plan->nnz, src, dst, out, D, plan->n_cols * int64_t{D} * 4,
+                                  plan->n_rows * int64_t{D} * 4, static_cast<hipStream_t>(stream));
 }
 
 int fg_sddmm_plan_describe(const fg_sddmm_plan *plan, int32_t H, int32_t D, char *buf, int64_t cap) {
@@ -487,7 +499,8 @@ int fg_config_set(const char *key, int32_t value) {
   const bool flag = slot == &fg::config().spmm_scalar_path || slot == &fg::config().spmm_sorted ||
                     slot == &fg::config().spmm_blocked || slot == &fg::config().spmm_pipeline ||
                     slot == &fg::config().spmm_sweep || slot == &fg::config().sddmm_blocked ||
-                    slot == &fg::config().spmm_buffer_loads;
+                    slot == &fg::config().spmm_buffer_loads || slot == &fg::config().sddmm_fast ||
+                    slot == &fg::config().sddmm_buffer_loads;
   // flags: 0 / 1 are explicit, anything negative restores the default;
   // sizes: 0 restores the default
   *slot = flag ? (value < 0 ? -1 : (value != 0)) : std::max(value, 0);

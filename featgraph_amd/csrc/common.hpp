@@ -26,6 +26,7 @@ struct Config {
   int spmm_blocked = -1, spmm_block_cols = 0, spmm_pipeline = -1, spmm_pipe_blocks = 0;
   int spmm_sweep = -1, spmm_sweep_waves_per_cu = 0, spmm_buffer_loads = -1;
   int sddmm_group = 0, sddmm_batches = 0, sddmm_blocked = -1, sddmm_block_cols = 0;
+  int sddmm_fast = -1, sddmm_buffer_loads = -1;
 };
 Config &config();
 
@@ -104,6 +105,7 @@ struct SddmmArgs {
   int32_t D;
   int32_t stride;  // floats per vertex row (= H * D)
   int32_t batches;  // 64-dot batches per wave
+  int64_t src_bytes = int64_t{1} << 40, dst_bytes = int64_t{1} << 40;  // extents of the two matrices
 };
 
 struct SddmmShape {
@@ -126,9 +128,14 @@ struct SddmmBlocks {
 int sddmm_blocks_build(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,
                        SddmmBlocks *out);
 void sddmm_blocks_free(SddmmBlocks *b);
-// src / dst 16-byte aligned, F a multiple of 4.
+// src / dst 16-byte aligned, F a multiple of 4; *_bytes: extents of the two matrices.
 int sddmm_blocked_launch(const SddmmBlocks &b, int64_t nnz, const float *src, const float *dst, float *out, int32_t F,
-                         hipStream_t stream);
+                         int64_t src_bytes, int64_t dst_bytes, hipStream_t stream);
+// One 64-float tile of every dot product of a (re-ordered) edge list: tile 0
+// stores to out[pos[i]], later tiles add to it (sddmm.hip).
+int sddmm_tile_launch(const int32_t *row_p, const int32_t *col_p, const int32_t *pos_p, int64_t nnz, const float *src,
+                      const float *dst, float *out, int64_t src_bytes, int64_t dst_bytes, int32_t F, int tile,
+                      hipStream_t stream);
 
 inline bool aligned_to(const void *p, uintptr_t bytes) { return (reinterpret_cast<uintptr_t>(p) & (bytes - 1)) == 0; }
 

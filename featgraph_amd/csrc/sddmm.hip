@@ -98,6 +98,122 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_kernel(const SddmmArgs a)
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// Fast path: float4 lanes, dot length D = G*4*CH exactly (or one 64-float tile
+// of a longer row), everything unrolled.  A wave takes 64 dot products; R
+// rounds (64/G dot products each) are issued together, so 2*R*CH float4 gathers
+// are in flight per lane before the first multiply, and no branch separates them.
+// With BUF the two matrices are addressed as buffer resources with 32-bit
+// per-lane byte offsets (one multiply-add per gather instead of 64-bit
+// arithmetic); that needs each matrix to span less than 4 GiB.
+struct FastArgs {
+  const int32_t *row;   // per dot product (plain: edge list; blocked: re-ordered list)
+  const int32_t *col;
+  const int32_t *pos;   // blocked: where each result goes; plain: null
+  const float *src;
+  const float *dst;
+  float *out;
+  int64_t n_ve;         // dot products (edges * heads)
+  int64_t src_bytes, dst_bytes;
+  int32_t H, D, stride;  // stride: floats per vertex row
+  int32_t first;         // first float of the row segment this launch covers (tile * 64)
+  int32_t valid;         // floats of the segment that exist (64, or fewer in the last tile)
+};
+
+template <bool BUF>
+struct VertexRows {
+  __amdgpu_buffer_rsrc_t rsrc;
+  const char *base;
+  __device__ __forceinline__ VertexRows(const float *p, int64_t bytes) : base(reinterpret_cast<const char *>(p)) {
+    rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p), 0,
+                                             BUF ? static_cast<int>(static_cast<uint32_t>(bytes)) : 0, 0x00020000);
+  }
+  // float4 at byte offset vertex * row_bytes + off
+  __device__ __forceinline__ float4 load(int vertex, uint32_t row_bytes, uint32_t off) const {
+    if constexpr (BUF) {
+      const uint32_t at = static_cast<uint32_t>(vertex) * row_bytes + off;
+      return __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, static_cast<int>(at), 0, 0));
+    } else {
+      return *reinterpret_cast<const float4 *>(base + static_cast<int64_t>(vertex) * row_bytes + off);
+    }
+  }
+};
+
+// MODE 0: plain (Out[v]), 1: blocked first tile (Out[pos] = sum), 2: blocked later tile (Out[pos] += sum)
+template <int G, int CH, bool MH, int MODE, bool BUF>
+__global__ __launch_bounds__(kBlockThreads) void sddmm_fast_kernel(const FastArgs a) {
+  constexpr int R = (8 / CH) < G ? (8 / CH) : G;  // rounds per batch: up to 16 float4 gathers in flight per lane
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int gl = lane & (G - 1);
+  const int gbase = lane & ~(G - 1);
+  const int64_t v_base = (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6)) * kWaveSize;
+  if (v_base >= a.n_ve) return;  // wave-uniform
+  const int64_t v = v_base + lane;
+  int my_row = 0, my_col = 0;  // lanes past the end gather vertex 0 and drop the result
+  int64_t my_pos = -1;
+  if (v < a.n_ve) {
+    const int64_t e = MH ? v / a.H : v;
+    my_row = a.row[e];
+    my_col = a.col[e];
+    my_pos = MODE == 0 ? v : a.pos[v];
+  }
+  float prev = 0.0f;
+  if (MODE == 2 && my_pos >= 0) prev = a.out[my_pos];
+  const VertexRows<BUF> src(a.src, a.src_bytes), dst(a.dst, a.dst_bytes);
+  const uint32_t row_bytes = static_cast<uint32_t>(a.stride) * 4u;
+  // this lane's float4 inside the segment; lanes past a short last tile re-read its last float4 and add zero
+  const bool kok = gl * 4 < a.valid;
+  const uint32_t lane_bytes = static_cast<uint32_t>(a.first + (kok ? gl * 4 : a.valid - 4)) * 4u;
+  float res = 0.0f;
+#pragma unroll
+  for (int jb = 0; jb < G; jb += R) {
+    float4 x[R][CH], y[R][CH];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int from = gbase + jb + r;
+      const int rr = __builtin_amdgcn_ds_bpermute(from << 2, my_row);
+      const int cc = __builtin_amdgcn_ds_bpermute(from << 2, my_col);
+      uint32_t off = lane_bytes;
+      if (MH) off += static_cast<uint32_t>((v_base + from) % a.H) * static_cast<uint32_t>(a.D) * 4u;
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        x[r][c] = src.load(cc, row_bytes, off + c * G * 16);
+        y[r][c] = dst.load(rr, row_bytes, off + c * G * 16);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float p = 0.0f;
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        p = __builtin_fmaf(x[r][c].x, y[r][c].x, p);
+        p = __builtin_fmaf(x[r][c].y, y[r][c].y, p);
+        p = __builtin_fmaf(x[r][c].z, y[r][c].z, p);
+        p = __builtin_fmaf(x[r][c].w, y[r][c].w, p);
+      }
+      p = kok ? p : 0.0f;
+      p = group_sum<G>(p);
+      if (gl == jb + r) res = p;
+    }
+  }
+  if (my_pos >= 0) a.out[my_pos] = MODE == 2 ? prev + res : res;
+}
+
+template <int G, int CH, bool MH, int MODE>
+int launch_fast_mode(const FastArgs &a, hipStream_t stream) {
+  const int64_t waves = (a.n_ve + kWaveSize - 1) / kWaveSize;
+  const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
+  if (blocks > 0x7fffffffLL) return fail(FG_EUNSUPPORTED, "SDDMM launch needs %lld blocks", (long long)blocks);
+  const bool buf = a.src_bytes < (int64_t{1} << 32) && a.dst_bytes < (int64_t{1} << 32) && config().sddmm_buffer_loads != 0;
+  if (buf)
+    sddmm_fast_kernel<G, CH, MH, MODE, true><<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(a);
+  else
+    sddmm_fast_kernel<G, CH, MH, MODE, false><<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(a);
+  FG_HIP_TRY(hipGetLastError());
+  return FG_OK;
+}
+
 template <int VEC, int G>
 int launch(const SddmmArgs &a, hipStream_t stream) {
   const int64_t per_wave = static_cast<int64_t>(a.batches) * kWaveSize;
@@ -142,8 +258,63 @@ SddmmShape sddmm_choose_shape(const SddmmArgs &a) {
   return s;
 }
 
+// Fast variant for this (H, D), or 1 when there is none.
+static int sddmm_launch_fast(const SddmmArgs &a, hipStream_t stream) {
+  if (a.D % 4 != 0 || !aligned_to(a.src, 16) || !aligned_to(a.dst, 16) || config().sddmm_fast == 0) return 1;
+  FastArgs f;
+  f.row = a.row;
+  f.col = a.col;
+  f.pos = nullptr;
+  f.src = a.src;
+  f.dst = a.dst;
+  f.out = a.out;
+  f.n_ve = a.n_ve;
+  f.src_bytes = a.src_bytes;
+  f.dst_bytes = a.dst_bytes;
+  f.H = a.H;
+  f.D = a.D;
+  f.stride = a.stride;
+  f.first = 0;
+  f.valid = a.D < 64 ? a.D : 64;
+  const bool mh = a.H > 1;
+  switch (a.D) {
+    case 16: return mh ? launch_fast_mode<4, 1, true, 0>(f, stream) : launch_fast_mode<4, 1, false, 0>(f, stream);
+    case 32: return mh ? launch_fast_mode<8, 1, true, 0>(f, stream) : launch_fast_mode<8, 1, false, 0>(f, stream);
+    case 64: return mh ? launch_fast_mode<16, 1, true, 0>(f, stream) : launch_fast_mode<16, 1, false, 0>(f, stream);
+    case 128: return mh ? launch_fast_mode<16, 2, true, 0>(f, stream) : launch_fast_mode<16, 2, false, 0>(f, stream);
+    case 256: return mh ? launch_fast_mode<16, 4, true, 0>(f, stream) : launch_fast_mode<16, 4, false, 0>(f, stream);
+    case 512: return mh ? launch_fast_mode<16, 8, true, 0>(f, stream) : launch_fast_mode<16, 8, false, 0>(f, stream);
+  }
+  return 1;
+}
+
+int sddmm_tile_launch(const int32_t *row_p, const int32_t *col_p, const int32_t *pos_p, int64_t nnz, const float *src,
+                      const float *dst, float *out, int64_t src_bytes, int64_t dst_bytes, int32_t F, int tile,
+                      hipStream_t stream) {
+  FastArgs f;
+  f.row = row_p;
+  f.col = col_p;
+  f.pos = pos_p;
+  f.src = src;
+  f.dst = dst;
+  f.out = out;
+  f.n_ve = nnz;
+  f.src_bytes = src_bytes;
+  f.dst_bytes = dst_bytes;
+  f.H = 1;
+  f.D = F;
+  f.stride = F;
+  f.first = tile * 64;
+  f.valid = F - tile * 64 < 64 ? F - tile * 64 : 64;
+  return tile == 0 ? launch_fast_mode<16, 1, false, 1>(f, stream) : launch_fast_mode<16, 1, false, 2>(f, stream);
+}
+
 int sddmm_launch(const SddmmArgs &a, const SddmmShape &s, hipStream_t stream) {
   if (a.n_ve == 0) return FG_OK;
+  if (config().sddmm_group == 0) {  // an explicit group size asks for the general kernel
+    const int rc = sddmm_launch_fast(a, stream);
+    if (rc != 1) return rc;
+  }
   SddmmArgs b = a;
   b.batches = s.batches;
   switch (s.vec) {

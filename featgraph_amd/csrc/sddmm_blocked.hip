@@ -29,12 +29,6 @@ namespace {
 
 constexpr int kTile = 64;  // floats per tile: 16 lanes x float4 per edge
 
-template <int CTRL>
-__device__ __forceinline__ float dpp_add(float x) {
-  const int y = __builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, false);
-  return x + __int_as_float(y);
-}
-
 __global__ void block_keys_kernel(const int32_t *col, int64_t nnz, int32_t block_cols, uint32_t *keys, int32_t *ids) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
@@ -51,63 +45,6 @@ __global__ void gather_edges_kernel(const int32_t *row, const int32_t *col, cons
     row_p[i] = row[e];
     col_p[i] = col[e];
   }
-}
-
-struct BlockedArgs {
-  const int32_t *row_p;
-  const int32_t *col_p;
-  const int32_t *pos_p;
-  const float *src;
-  const float *dst;
-  float *out;
-  int64_t nnz;
-  int32_t F;
-  int32_t tile;
-};
-
-// 64 edges per wave; 16 lanes x float4 cover one 64-float tile of one edge, so
-// four edges are in flight per round and 16 rounds finish the wave's 64 edges.
-template <bool ACC>
-__global__ __launch_bounds__(kBlockThreads) void sddmm_blocked_kernel(const BlockedArgs a) {
-  const int lane = threadIdx.x & (kWaveSize - 1);
-  const int gl = lane & 15;
-  const int gbase = lane & ~15;
-  const int64_t base = (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6)) * kWaveSize;
-  if (base >= a.nnz) return;
-  const int64_t i = base + lane;
-  int my_row = 0, my_col = 0, my_pos = -1;
-  if (i < a.nnz) {
-    my_row = a.row_p[i];
-    my_col = a.col_p[i];
-    my_pos = a.pos_p[i];
-  }
-  float prev = 0.0f;
-  if (ACC && my_pos >= 0) prev = a.out[my_pos];
-  const int k = a.tile * kTile + gl * 4;
-  const bool kok = k < a.F;
-  const int64_t F = a.F;
-  float res = 0.0f;
-#pragma unroll 8
-  for (int j = 0; j < 16; ++j) {
-    const int from = gbase + j;
-    const int r = __builtin_amdgcn_ds_bpermute(from << 2, my_row);
-    const int c = __builtin_amdgcn_ds_bpermute(from << 2, my_col);
-    float p = 0.0f;
-    if (kok) {
-      const float4 x = *reinterpret_cast<const float4 *>(a.src + static_cast<int64_t>(c) * F + k);
-      const float4 y = *reinterpret_cast<const float4 *>(a.dst + static_cast<int64_t>(r) * F + k);
-      p = __builtin_fmaf(x.x, y.x, p);
-      p = __builtin_fmaf(x.y, y.y, p);
-      p = __builtin_fmaf(x.z, y.z, p);
-      p = __builtin_fmaf(x.w, y.w, p);
-    }
-    p = dpp_add<0xB1>(p);   // quad_perm [1,0,3,2]
-    p = dpp_add<0x4E>(p);   // quad_perm [2,3,0,1]
-    p = dpp_add<0x141>(p);  // row_half_mirror
-    p = dpp_add<0x140>(p);  // row_mirror
-    if (gl == j) res = p;
-  }
-  if (my_pos >= 0) a.out[my_pos] = ACC ? prev + res : res;
 }
 
 }  // namespace
@@ -179,28 +116,11 @@ int sddmm_blocks_build(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_
 }
 
 int sddmm_blocked_launch(const SddmmBlocks &b, int64_t nnz, const float *src, const float *dst, float *out, int32_t F,
-                         hipStream_t stream) {
-  BlockedArgs a;
-  a.row_p = b.row_p;
-  a.col_p = b.col_p;
-  a.pos_p = b.pos_p;
-  a.src = src;
-  a.dst = dst;
-  a.out = out;
-  a.nnz = nnz;
-  a.F = F;
-  const int64_t waves = (nnz + kWaveSize - 1) / kWaveSize;
-  const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
-  if (blocks > 0x7fffffffLL) return fail(FG_EUNSUPPORTED, "SDDMM launch needs %lld blocks", (long long)blocks);
+                         int64_t src_bytes, int64_t dst_bytes, hipStream_t stream) {
   const int n_tiles = (F + kTile - 1) / kTile;
-  for (int t = 0; t < n_tiles; ++t) {
-    a.tile = t;
-    if (t == 0)
-      sddmm_blocked_kernel<false><<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(a);
-    else
-      sddmm_blocked_kernel<true><<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(a);
-    FG_HIP_TRY(hipGetLastError());
-  }
+  for (int t = 0; t < n_tiles; ++t)
+    if (int rc = sddmm_tile_launch(b.row_p, b.col_p, b.pos_p, nnz, src, dst, out, src_bytes, dst_bytes, F, t, stream))
+      return rc;
   return FG_OK;
 }
 

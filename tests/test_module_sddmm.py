@@ -31,7 +31,8 @@ def config_guard():
     _lib.config_set("sddmm.group", 0)
     _lib.config_set("sddmm.batches", 0)
     _lib.config_set("sddmm.block_cols", 0)
-    _lib.config_set("sddmm.blocked", -1)
+    for key in ("sddmm.blocked", "sddmm.fast", "sddmm.buffer_loads"):
+        _lib.config_set(key, -1)
 
 
 # the reference's own test on its matrix family (tests/test_module_sddmm.py:44-70)
@@ -177,6 +178,28 @@ def test_column_blocked_falls_back_for_odd_lengths_and_heads(config_guard):
     src, dst = datasets.sddmm_operands(coo, (4, 16))
     out = _run_sddmm(coo, src, dst, cls=MultiHeadSDDMMhip)
     np.testing.assert_allclose(out, ref.sddmm_mh(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("shape", [(1, 16), (1, 32), (1, 64), (1, 128), (1, 256), (1, 512), (8, 16), (8, 32), (8, 64),
+                                   (3, 128)])
+def test_unrolled_kernel_against_the_general_one(config_guard, shape):
+    H, D = shape
+    coo = datasets.config_graph("c4-mini").tocoo()
+    cls = VanillaSDDMMhip if H == 1 else MultiHeadSDDMMhip
+    src, dst = datasets.sddmm_operands(coo, D if H == 1 else (H, D))
+    want = ref.sddmm_mh(coo.row, coo.col, src.reshape(-1, H, D), dst.reshape(-1, H, D)).reshape(-1) if H > 1 \
+        else ref.sddmm_x86(coo.row, coo.col, src, dst)
+    _lib.config_set("sddmm.blocked", 0)
+    outs = {}
+    for fast, buf in ((0, 0), (1, 0), (1, 1)):
+        _lib.config_set("sddmm.fast", fast)
+        _lib.config_set("sddmm.buffer_loads", buf)
+        out = _run_sddmm(coo, src, dst, cls=cls).reshape(-1)
+        np.testing.assert_allclose(out, want, rtol=RTOL, atol=ATOL)
+        outs[(fast, buf)] = out
+    assert np.array_equal(outs[(1, 0)], outs[(1, 1)])               # addressing mode cannot change a bit
+    if D <= 64:
+        assert np.array_equal(outs[(0, 0)], outs[(1, 0)])           # one step per lane: same summation tree
 
 
 def test_module_surface(adj_127x255):
