@@ -161,7 +161,9 @@ def main():
             args.graph, n_rows, nnz, F), "graph_checksum": datasets.structure_checksum(adj)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": committed_traffic("spmm", F),
-                     "algorithmic_bytes": alg, "kernel": "spmm (CSR, feat-len %d)" % F, "launch_ms": ms},
+                     "algorithmic_bytes": alg, "kernel": "spmm (CSR, feat-len %d)" % F, "launch_ms": ms,
+                     "note": "one operator launch may be several dispatches of the same kernel (one per column "
+                             "block and feature tile, see `launch`); bytes, time and traffic are per operator launch"},
         "launch": spmm.lower_to_ir([placeholder((n_cols, F))], {}, {}),
     }
     if args.only == "spmm":

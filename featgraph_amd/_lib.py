@@ -16,6 +16,7 @@ SIGNATURES = {
     "fg_version": (ctypes.c_int, []),
     "fg_last_error": (ctypes.c_char_p, []),
     "fg_spmm_plan_create": (ctypes.c_int, [_i64, _i64, _i64, _p, _p, ctypes.POINTER(_p)]),
+    "fg_spmm_plan_create_partitioned": (ctypes.c_int, [_i64, _i64, _i64, _p, _p, _i32, ctypes.POINTER(_p)]),
     "fg_spmm_plan_destroy": (None, [_p]),
     "fg_spmm_plan_row_order": (ctypes.c_int, [_p, _p, ctypes.POINTER(_i32)]),
     "fg_spmm_csr_f32": (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _p]),
@@ -23,6 +24,7 @@ SIGNATURES = {
     "fg_sddmm_coo_f32": (ctypes.c_int, [_i64, _p, _p, _p, _p, _p, _i32, _p]),
     "fg_sddmm_coo_mh_f32": (ctypes.c_int, [_i64, _p, _p, _p, _p, _p, _i32, _i32, _p]),
     "fg_sddmm_plan_create": (ctypes.c_int, [_i64, _i64, _i64, _p, _p, ctypes.POINTER(_p)]),
+    "fg_sddmm_plan_create_partitioned": (ctypes.c_int, [_i64, _i64, _i64, _p, _p, _i32, ctypes.POINTER(_p)]),
     "fg_sddmm_plan_destroy": (None, [_p]),
     "fg_sddmm_coo_plan_f32": (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _p]),
     "fg_sddmm_plan_describe": (ctypes.c_int, [_p, _i32, _i32, ctypes.c_char_p, _i64]),

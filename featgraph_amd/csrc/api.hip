@@ -47,6 +47,8 @@ struct fg_spmm_plan {
   int32_t *seg;  // owned, device, (n_blocks + 1) * n_rows entries
   int32_t n_blocks;
   int32_t block_cols;
+  int32_t requested_partitions;  // 0: library decides; 1: no column blocks; P > 1: P blocks, as the caller asked
+  bool force_blocks;             // the caller's P > 1: use the blocks at every feature length
   fg::SweepPlan sweep;  // per-wave block-major lists (optional)
 };
 
@@ -54,6 +56,7 @@ struct fg_sddmm_plan {
   int64_t nnz, n_rows, n_cols;
   const int32_t *row;  // borrowed, device
   const int32_t *col;  // borrowed, device
+  bool force_blocks;   // the caller asked for column partitions: use them at every feature length
   fg::SddmmBlocks blocks;
 };
 
@@ -132,7 +135,9 @@ bool use_sweep(const fg_spmm_plan *plan, const fg::SpmmArgs &a) {
 }
 
 bool use_column_blocks(const fg_spmm_plan *plan, const fg::SpmmArgs &a, const fg::SpmmShape &s) {
-  if (!plan->seg || plan->n_blocks < 2 || !a.row_order || fg::config().spmm_blocked == 0) return false;
+  if (!plan->seg || plan->n_blocks < 2 || !a.row_order) return false;
+  if (plan->force_blocks) return true;
+  if (fg::config().spmm_blocked == 0) return false;
   if (fg::config().spmm_blocked > 0) return true;
   // worthwhile only while the whole gathered band does not fit an L2 anyway
   const int64_t band_bytes = static_cast<int64_t>(plan->n_cols) * std::min<int64_t>(s.tile_width(), a.F) * 4;
@@ -172,10 +177,16 @@ int build_bounds(fg_spmm_plan *p) {
   const fg::Config &cfg = fg::config();
   if (p->n_rows == 0) return FG_OK;
   int64_t block_cols = cfg.spmm_block_cols > 0 ? cfg.spmm_block_cols : 16384;
-  int64_t n_blocks = (p->n_cols + block_cols - 1) / block_cols;
+  const int P = p->requested_partitions;
+  if (P > 1) block_cols = std::max<int64_t>(1, (p->n_cols + P - 1) / P);  // util/adj_partitioning.py:42
+  int64_t n_blocks = p->n_cols > 0 ? (p->n_cols + block_cols - 1) / block_cols : 1;
   const double per_segment =
       n_blocks > 0 ? static_cast<double>(p->nnz) / (static_cast<double>(p->n_rows) * n_blocks) : 0.0;
-  if (cfg.spmm_blocked == 0 || n_blocks < 2 || (cfg.spmm_blocked < 0 && per_segment < 8.0)) n_blocks = 1;
+  if (P == 1 || n_blocks < 2 || p->nnz == 0)
+    n_blocks = 1;
+  else if (P == 0 && (cfg.spmm_blocked == 0 || (cfg.spmm_blocked < 0 && per_segment < 8.0)))
+    n_blocks = 1;
+  p->force_blocks = P > 1;
   int *flag = nullptr;
   FG_HIP_TRY(hipMalloc(&flag, sizeof(int)));
   for (;;) {
@@ -274,8 +285,15 @@ const char *fg_last_error(void) { return fg::g_error; }
 
 int fg_spmm_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr, const int32_t *indices,
                         fg_spmm_plan **plan) {
+  return fg_spmm_plan_create_partitioned(n_rows, n_cols, nnz, indptr, indices, 0, plan);
+}
+
+int fg_spmm_plan_create_partitioned(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr,
+                                    const int32_t *indices, int32_t num_col_partitions, fg_spmm_plan **plan) {
   if (!plan) return fg::fail(FG_EINVAL, "plan output pointer is null");
   *plan = nullptr;
+  if (num_col_partitions < 0)
+    return fg::fail(FG_EINVAL, "num_col_partitions = %d is negative", num_col_partitions);
   if (n_rows < 0 || n_cols < 0 || nnz < 0)
     return fg::fail(FG_EINVAL, "negative size (n_rows=%lld n_cols=%lld nnz=%lld)", (long long)n_rows,
                     (long long)n_cols, (long long)nnz);
@@ -318,6 +336,8 @@ int fg_spmm_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32
   p->indptr = indptr;
   p->indices = indices;
   p->row_order = nullptr;
+  p->requested_partitions = num_col_partitions;
+  p->force_blocks = false;
   p->max_degree = max_degree;
   p->device = 0;
   hipError_t err = hipGetDevice(&p->device);
@@ -405,8 +425,15 @@ int fg_sddmm_coo_mh_f32(int64_t nnz, const int32_t *row, const int32_t *col, con
 
 int fg_sddmm_plan_create(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,
                          fg_sddmm_plan **plan) {
+  return fg_sddmm_plan_create_partitioned(nnz, n_rows, n_cols, row, col, 0, plan);
+}
+
+int fg_sddmm_plan_create_partitioned(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row,
+                                     const int32_t *col, int32_t num_col_partitions, fg_sddmm_plan **plan) {
   if (!plan) return fg::fail(FG_EINVAL, "plan output pointer is null");
   *plan = nullptr;
+  if (num_col_partitions < 0)
+    return fg::fail(FG_EINVAL, "num_col_partitions = %d is negative", num_col_partitions);
   if (nnz < 0 || n_rows < 0 || n_cols < 0)
     return fg::fail(FG_EINVAL, "negative size (nnz=%lld n_rows=%lld n_cols=%lld)", (long long)nnz, (long long)n_rows,
                     (long long)n_cols);
@@ -419,7 +446,8 @@ int fg_sddmm_plan_create(int64_t nnz, int64_t n_rows, int64_t n_cols, const int3
   p->n_cols = n_cols;
   p->row = row;
   p->col = col;
-  if (int rc = fg::sddmm_blocks_build(nnz, n_rows, n_cols, row, col, &p->blocks)) {
+  p->force_blocks = num_col_partitions > 1;
+  if (int rc = fg::sddmm_blocks_build(nnz, n_rows, n_cols, row, col, num_col_partitions, &p->blocks)) {
     delete p;
     return rc;
   }
@@ -435,8 +463,8 @@ void fg_sddmm_plan_destroy(fg_sddmm_plan *plan) {
 
 static bool sddmm_use_blocks(const fg_sddmm_plan *plan, const float *src, const float *dst, int32_t H, int32_t D) {
   // below 64 floats a tile would leave lanes idle and the plain kernel is as fast (measured at 32)
-  if (fg::config().sddmm_blocked < 0 && D < 64) return false;
-  return plan->blocks.pos_p && fg::config().sddmm_blocked != 0 && H == 1 && D % 4 == 0 && fg::aligned_to(src, 16) &&
+  if (!plan->force_blocks && (fg::config().sddmm_blocked == 0 || (fg::config().sddmm_blocked < 0 && D < 64))) return false;
+  return plan->blocks.pos_p && H == 1 && D % 4 == 0 && fg::aligned_to(src, 16) &&
          fg::aligned_to(dst, 16);
 }
 
@@ -536,7 +564,9 @@ int fg_spmm_describe(const fg_spmm_plan *plan, int32_t H, int32_t D, int32_t fea
   const int rows_per_wave = fg::kWaveSize / s.lpr;
   const bool blocked = use_column_blocks(plan, a, s);
   const int64_t slots = blocked ? a.n_rows : a.n_slots;
-  const int64_t waves = (slots + rows_per_wave - 1) / rows_per_wave;
+  int64_t waves = (slots + rows_per_wave - 1) / rows_per_wave;
+  if (s.pipeline)  // a fixed grid whose waves each walk several rows
+    waves = std::min<int64_t>(waves, static_cast<int64_t>(s.pipe_blocks) * fg::kWavesPerBlock);
   char passes[96] = "1 launch";
   if (blocked)
     snprintf(passes, sizeof(passes), "%d launches (%d tiles x %d column blocks of %d)", a.n_tiles * plan->n_blocks,

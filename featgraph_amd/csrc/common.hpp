@@ -125,8 +125,9 @@ struct SddmmBlocks {
   int32_t block_cols = 0;
 };
 
+// num_col_partitions: 0 lets the library decide, 1 builds nothing, P > 1 builds P column blocks.
 int sddmm_blocks_build(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,
-                       SddmmBlocks *out);
+                       int32_t num_col_partitions, SddmmBlocks *out);
 void sddmm_blocks_free(SddmmBlocks *b);
 // src / dst 16-byte aligned, F a multiple of 4; *_bytes: extents of the two matrices.
 int sddmm_blocked_launch(const SddmmBlocks &b, int64_t nnz, const float *src, const float *dst, float *out, int32_t F,

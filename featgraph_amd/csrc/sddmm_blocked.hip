@@ -57,15 +57,20 @@ void sddmm_blocks_free(SddmmBlocks *b) {
 }
 
 int sddmm_blocks_build(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,
-                       SddmmBlocks *out) {
+                       int32_t num_col_partitions, SddmmBlocks *out) {
   *out = SddmmBlocks();
   const Config &cfg = config();
-  if (cfg.sddmm_blocked == 0 || nnz == 0 || n_rows == 0 || nnz > 0x7fffffffLL) return FG_OK;
-  const int64_t block_cols = cfg.sddmm_block_cols > 0 ? cfg.sddmm_block_cols : 16384;
+  if (num_col_partitions == 1 || nnz == 0 || n_rows == 0 || n_cols == 0 || nnz > 0x7fffffffLL) return FG_OK;
+  if (num_col_partitions == 0 && cfg.sddmm_blocked == 0) return FG_OK;
+  int64_t block_cols = cfg.sddmm_block_cols > 0 ? cfg.sddmm_block_cols : 16384;
+  if (num_col_partitions > 1)  // the caller's count, block width as in util/adj_partitioning.py:98
+    block_cols = std::max<int64_t>(1, (n_cols + num_col_partitions - 1) / num_col_partitions);
   const int64_t n_blocks = (n_cols + block_cols - 1) / block_cols;
   if (n_blocks < 2) return FG_OK;
-  // worthwhile while a destination row still meets several of its edges inside one block
-  if (cfg.sddmm_blocked < 0 && static_cast<double>(nnz) / (static_cast<double>(n_rows) * n_blocks) < 4.0) return FG_OK;
+  // on its own the library blocks only while a destination row still meets several of its edges inside one block
+  if (num_col_partitions == 0 && cfg.sddmm_blocked < 0 &&
+      static_cast<double>(nnz) / (static_cast<double>(n_rows) * n_blocks) < 4.0)
+    return FG_OK;
   int bits = 1;
   while ((int64_t{1} << bits) < n_blocks) ++bits;
 

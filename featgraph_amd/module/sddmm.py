@@ -35,15 +35,18 @@ def normalize_coo(adj_scipy):
 class SDDMMbase:
     """Base class of the SDDMM-like modules (reference: module/sddmm.py:11-165)."""
 
-    def __init__(self, adj_scipy, num_row_partitions=1, num_col_partitions=1):
-        assert num_row_partitions >= 1, "num_row_partitions should be larger than or equal to 1"
-        assert num_col_partitions >= 1, "num_col_partitions should be larger than or equal to 1"
-        if num_row_partitions != 1 or num_col_partitions != 1:
-            raise NotImplementedError("2-D graph partitioning is a CPU cache-blocking scheme of the x86 target; "
-                                      "the HIP target takes no partition counts")
+    def __init__(self, adj_scipy, num_row_partitions=None, num_col_partitions=None):
+        """Partition counts as in the reference (module/sddmm.py:13-26).  On this target cache blocking is by
+        column blocks only (the row dimension is already local in a row-sorted edge list): num_col_partitions
+        None lets the library decide, 1 turns blocking off, P > 1 asks for P blocks; num_row_partitions is
+        checked and otherwise unused.  Outputs always come in the caller's edge order."""
+        if num_row_partitions is not None:
+            assert num_row_partitions >= 1, "num_row_partitions should be larger than or equal to 1"
+        if num_col_partitions is not None:
+            assert num_col_partitions >= 1, "num_col_partitions should be larger than or equal to 1"
         row, col, (self._num_rows, self._num_cols) = normalize_coo(adj_scipy)
-        self._num_row_partitions = 1
-        self._num_col_partitions = 1
+        self._num_row_partitions = num_row_partitions or 1
+        self._num_col_partitions = num_col_partitions or 1
         self._nnz = int(row.shape[0])
         self._target = None
         self._ctx = None
@@ -55,9 +58,9 @@ class SDDMMbase:
         # (module/sddmm.py:45-49) is a column-block plan on the device here; outputs stay in edge order
         self._plan = ctypes.c_void_p()
         with torch.cuda.device(self._ctx):
-            _lib.check(_lib.lib().fg_sddmm_plan_create(
+            _lib.check(_lib.lib().fg_sddmm_plan_create_partitioned(
                 self._nnz, self._num_rows, self._num_cols, self._adj_row_dev.data_ptr(),
-                self._adj_col_dev.data_ptr(), ctypes.byref(self._plan)))
+                self._adj_col_dev.data_ptr(), int(num_col_partitions or 0), ctypes.byref(self._plan)))
         self._built = False
         self.out_tvm = None
 
@@ -150,11 +153,12 @@ class SDDMMbase:
 
     @property
     def edge_mapping(self):
-        # module/sddmm.py:152-157: only the partitioned x86 path has one
-        assert self._target not in ("cuda", "hip"), "no graph partitioning on %s, no edge_mapping" % self._target
+        """Permutation that puts run() results back into the caller's edge order (module/sddmm.py:152-157,
+        tests/test_module_sddmm.py:31-32).  Results here are already in that order, so it is the identity;
+        like the reference it exists only when partitioning was asked for."""
         assert self._num_row_partitions > 1 or self._num_col_partitions > 1, \
             "no graph partitioning, no edge_mapping"
-        return None
+        return np.arange(self._nnz)
 
     @property
     def ctx(self):
@@ -166,10 +170,11 @@ class SDDMMbase:
 
 
 class VanillaSDDMMhip(SDDMMbase):
-    """COO SDDMM on the GPU; constructor signature of VanillaSDDMMcuda (module/sddmm.py:179-181)."""
+    """COO SDDMM on the GPU.  VanillaSDDMMhip(adj) is the call of VanillaSDDMMcuda (module/sddmm.py:179-181);
+    the optional partition counts are the arguments of VanillaSDDMMx86 (:169)."""
 
-    def __init__(self, adj_scipy):
-        super().__init__(adj_scipy, num_row_partitions=1, num_col_partitions=1)
+    def __init__(self, adj_scipy, num_row_partitions=None, num_col_partitions=None):
+        super().__init__(adj_scipy, num_row_partitions, num_col_partitions)
 
     def _register(self):
         self._target = "hip"
@@ -183,7 +188,7 @@ class MultiHeadSDDMMhip(SDDMMbase):
     """
 
     def __init__(self, adj_scipy):
-        super().__init__(adj_scipy, num_row_partitions=1, num_col_partitions=1)
+        super().__init__(adj_scipy)
 
     def _register(self):
         self._target = "hip"

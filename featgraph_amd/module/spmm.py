@@ -47,13 +47,14 @@ class SpMMbase:
 
     _input_names = ("SrcFeat",)
 
-    def __init__(self, adj_scipy, num_col_partitions=1):
-        assert num_col_partitions >= 1, "num_col_partitions should be larger than or equal to 1"
-        if num_col_partitions != 1:
-            raise NotImplementedError("source-vertex partitioning is a CPU cache-blocking scheme of the x86 target; "
-                                      "the HIP target takes num_col_partitions=1")
+    def __init__(self, adj_scipy, num_col_partitions=None):
+        """num_col_partitions: the reference's 1-D source-vertex partitioning (module/spmm.py:14-24).  On this
+        target it selects the number of column blocks of the L2-blocked passes: None lets the library decide
+        from the matrix, 1 turns blocking off, P > 1 asks for P blocks.  It never changes a result bit."""
+        if num_col_partitions is not None:
+            assert num_col_partitions >= 1, "num_col_partitions should be larger than or equal to 1"
         indptr, indices, data, (self._num_rows, self._num_cols) = normalize_csr(adj_scipy)
-        self._num_col_partitions = 1
+        self._num_col_partitions = num_col_partitions
         self._nnz = int(indices.shape[0])
         self._target = None
         self._ctx = None
@@ -65,9 +66,9 @@ class SpMMbase:
         self._adj_vals_dev = torch.from_numpy(data).to(self._ctx)
         self._plan = ctypes.c_void_p()
         with torch.cuda.device(self._ctx):
-            _lib.check(_lib.lib().fg_spmm_plan_create(
+            _lib.check(_lib.lib().fg_spmm_plan_create_partitioned(
                 self._num_rows, self._num_cols, self._nnz, self._adj_indptr_dev.data_ptr(),
-                self._adj_indices_dev.data_ptr(), ctypes.byref(self._plan)))
+                self._adj_indices_dev.data_ptr(), int(num_col_partitions or 0), ctypes.byref(self._plan)))
         self._feat_shape = None
         self._feat_tiles = 0
         self._built = False
@@ -186,10 +187,11 @@ class SpMMbase:
 
 
 class VanillaSpMMhip(SpMMbase):
-    """CSR SpMM on the GPU; constructor signature of VanillaSpMMcuda (module/spmm.py:212-214)."""
+    """CSR SpMM on the GPU.  VanillaSpMMhip(adj) is the call of VanillaSpMMcuda (module/spmm.py:212-214);
+    the optional num_col_partitions is the argument of VanillaSpMMx86 (:198)."""
 
-    def __init__(self, adj_scipy):
-        super().__init__(adj_scipy, num_col_partitions=1)
+    def __init__(self, adj_scipy, num_col_partitions=None):
+        super().__init__(adj_scipy, num_col_partitions)
 
     def _register(self):
         self._target = "hip"
@@ -207,8 +209,8 @@ class MultiHeadSpMMhip(SpMMbase):
 
     _input_names = ("SrcFeat", "EdgeWeight")
 
-    def __init__(self, adj_scipy):
-        super().__init__(adj_scipy, num_col_partitions=1)
+    def __init__(self, adj_scipy, num_col_partitions=None):
+        super().__init__(adj_scipy, num_col_partitions)
 
     def _register(self):
         self._target = "hip"

@@ -64,6 +64,15 @@ FG_API const char *fg_last_error(void);
  */
 FG_API int fg_spmm_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr,
                         const int32_t *indices, fg_spmm_plan **plan);
+/*
+ * The same with the caller's say on column blocking, the num_col_partitions of
+ * VanillaSpMMx86 (module/spmm.py:198, util/adj_partitioning.py:42): 0 = as
+ * fg_spmm_plan_create, 1 = no column blocks, P > 1 = P blocks of
+ * ceil(n_cols / P) columns, used at every feature length (rows whose column ids
+ * do not ascend still fall back to a single pass).  Never changes a result bit.
+ */
+FG_API int fg_spmm_plan_create_partitioned(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr,
+                                           const int32_t *indices, int32_t num_col_partitions, fg_spmm_plan **plan);
 FG_API void fg_spmm_plan_destroy(fg_spmm_plan *plan);
 
 /* Copies the plan's row order (n_rows int32) to HOST memory at row_order_host
@@ -116,6 +125,10 @@ FG_API int fg_sddmm_coo_f32(int64_t nnz, const int32_t *row, const int32_t *col,
 typedef struct fg_sddmm_plan fg_sddmm_plan;
 FG_API int fg_sddmm_plan_create(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,
                                 fg_sddmm_plan **plan);
+/* The same with the caller's num_col_partitions (module/sddmm.py:169): 0 = library decides, 1 = no blocks,
+ * P > 1 = P blocks of ceil(n_cols / P) columns. */
+FG_API int fg_sddmm_plan_create_partitioned(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row,
+                                            const int32_t *col, int32_t num_col_partitions, fg_sddmm_plan **plan);
 FG_API void fg_sddmm_plan_destroy(fg_sddmm_plan *plan);
 
 /*

@@ -108,3 +108,19 @@ def test_c5_multihead_spmm_d64(c4):
     out = module.run([nd.array(feat, module.ctx), nd.array(w, module.ctx)]).asnumpy()
     want = ref.spmm_mh(adj.indptr, adj.indices, w, feat)
     assert np.array_equal(out, want)
+
+
+def test_benchmark_commands_run_on_a_small_graph(tmp_path, capsys):
+    import scipy.sparse
+    from featgraph_amd.benchmark import bench_vanilla_sddmm, bench_vanilla_spmm
+    adj = datasets.config_graph("c2-mini")
+    path = str(tmp_path / "adj_csr.npz")
+    scipy.sparse.save_npz(path, adj)                       # the .npz layout the reference's --dataset flag reads
+    args = bench_vanilla_spmm.C.parser("t", "csr").parse_args(["--dataset", path, "--feat-len", "32"])
+    loaded = bench_vanilla_spmm.C.load_adjacency(args, "csr")
+    assert loaded.format == "csr" and loaded.nnz == adj.nnz
+    res = bench_vanilla_spmm.bench_vanilla_spmm_hip(loaded, args.feat_len, 2)
+    assert len(res) == 7 * 3 and all(t > 0 for t, _ in res)
+    res = bench_vanilla_sddmm.bench_vanilla_sddmm_hip(adj.tocoo(), 32, 2)
+    assert len(res) == 7 and all(t > 0 for t, _ in res)
+    assert "best:" in capsys.readouterr().out

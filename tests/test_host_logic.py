@@ -90,6 +90,8 @@ def test_partition_counts_are_asserted_like_the_reference():
         SpMMbase(adj, num_col_partitions=0)
     with pytest.raises(AssertionError):
         SDDMMbase(adj, num_row_partitions=0)
+    with pytest.raises(AssertionError):
+        SDDMMbase(adj, num_col_partitions=0)
 
 
 def test_package_does_not_import_the_checker():

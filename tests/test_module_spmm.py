@@ -53,6 +53,24 @@ def test_vanilla_spmm_hip_like_the_reference_cuda_test(adj_127x255, num_threads_
     assert np.array_equal(out, _oracle(adj, feat))
 
 
+# its x86 test's partition arguments (tests/test_module_spmm.py:16-34): (feat_len, num_col_partitions, num_feat_partitions)
+@pytest.mark.parametrize("num_col_partitions,num_feat_partitions", [(1, 1), (4, 1), (4, 4), (300, 2)])
+def test_partition_arguments_like_the_reference_x86_test(adj_127x255, num_col_partitions, num_feat_partitions):
+    adj = adj_127x255
+    feat = np.random.default_rng(3).random((adj.shape[1], 128)).astype("float32")
+    module = VanillaSpMMhip(adj, num_col_partitions)
+    module.build([placeholder(feat.shape)], {"num_feat_partitions": num_feat_partitions}, {})
+    text = module.lower_to_ir([placeholder(feat.shape)], {"num_feat_partitions": num_feat_partitions}, {})
+    assert ("column blocks" in text) == (num_col_partitions > 1)
+    out = module.run([nd.array(feat, module.ctx)]).asnumpy()
+    np.testing.assert_allclose(adj.dot(feat), out, rtol=1e-4, atol=1e-4)
+    assert np.array_equal(out, _oracle(adj, feat, num_feat_partitions))
+    # the reference's DDS nest re-associates the sum per block; the kernel stays within tolerance of it too
+    s1_pos, s1_idx, vals = __import__("featgraph_amd").util.util_convert_csr_to_dds(adj, min(num_col_partitions, 8))
+    dds = ref.spmm_dds_x86(s1_pos, s1_idx, vals, feat, adj.shape[0], min(num_col_partitions, 8), num_feat_partitions)
+    np.testing.assert_allclose(out, dds, rtol=RTOL, atol=ATOL)
+
+
 # ... and its x86 test's feature-partition arguments (:32-34)
 @pytest.mark.parametrize("num_feat_partitions", [1, 4, 8])
 def test_feature_partitions_never_change_a_bit(adj_127x255, num_feat_partitions):
