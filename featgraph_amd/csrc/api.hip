@@ -49,6 +49,11 @@ struct fg_spmm_plan {
   int32_t block_cols;
   int32_t requested_partitions;  // 0: library decides; 1: no column blocks; P > 1: P blocks, as the caller asked
   bool force_blocks;             // the caller's P > 1: use the blocks at every feature length
+  // what the bounds table is built from: block width (0: default), blocks on / off / automatic (1 / 0 / -1),
+  // and the nonzeros per (row, block) below which automatic mode keeps whole rows
+  int32_t want_block_cols;
+  int want_blocked;
+  double min_per_segment;
   fg::SweepPlan sweep;  // per-wave block-major lists (optional)
 };
 
@@ -58,7 +63,15 @@ struct fg_sddmm_plan {
   const int32_t *col;  // borrowed, device
   bool force_blocks;   // the caller asked for column partitions: use them at every feature length
   fg::SddmmBlocks blocks;
+  // Row-sorted lists (a COO list derived from CSR): the row pointer rebuilt from `row`, and a row plan over
+  // it (visiting order + per-column-block bounds) for the row-run kernel.  Null otherwise.
+  int32_t *indptr = nullptr;      // owned, device, n_rows + 1 entries
+  fg_spmm_plan *rows = nullptr;   // owned
 };
+
+static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr, const int32_t *indices,
+                           int32_t num_col_partitions, int32_t want_block_cols, int want_blocked,
+                           double min_per_segment, bool with_sweep, fg_spmm_plan **plan);
 
 namespace {
 
@@ -90,6 +103,28 @@ __global__ void build_segments_kernel(const int32_t *indptr, const int32_t *indi
       if (e < end && indices[e - 1] > indices[e]) atomicOr(unsorted, 1);
     }
     for (int b = bp + 1; b <= bk; ++b) seg[static_cast<int64_t>(b) * n_rows + i] = e;
+  }
+}
+
+// Raises *bad when the row ids of an edge list descend somewhere or leave [0, n_rows).
+__global__ void rows_sorted_kernel(const int32_t *row, int64_t nnz, int32_t n_rows, int *bad) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  int b = 0;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
+    const int32_t r = row[i];
+    b |= (r < 0 || r >= n_rows) ? 1 : 0;
+    if (i + 1 < nnz) b |= row[i + 1] < r ? 1 : 0;
+  }
+  if (b) atomicOr(bad, 1);
+}
+
+// Row pointer of a row-sorted edge list: indptr[r] = number of edges whose row id is below r.
+__global__ void indptr_from_rows_kernel(const int32_t *row, int64_t nnz, int32_t n_rows, int32_t *indptr) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i <= nnz; i += stride) {
+    const int32_t prev = i > 0 ? row[i - 1] : -1;
+    const int32_t cur = i < nnz ? row[i] : n_rows;
+    for (int32_t r = prev + 1; r <= cur; ++r) indptr[r] = static_cast<int32_t>(i);
   }
 }
 
@@ -174,9 +209,8 @@ int sddmm_prepare(int64_t nnz, const int32_t *row, const int32_t *col, const flo
 // matrix does not, and when a row still has enough nonzeros per block to
 // amortise re-reading its partial sum; otherwise the table holds whole rows.
 int build_bounds(fg_spmm_plan *p) {
-  const fg::Config &cfg = fg::config();
   if (p->n_rows == 0) return FG_OK;
-  int64_t block_cols = cfg.spmm_block_cols > 0 ? cfg.spmm_block_cols : 16384;
+  int64_t block_cols = p->want_block_cols > 0 ? p->want_block_cols : 16384;
   const int P = p->requested_partitions;
   if (P > 1) block_cols = std::max<int64_t>(1, (p->n_cols + P - 1) / P);  // util/adj_partitioning.py:42
   int64_t n_blocks = p->n_cols > 0 ? (p->n_cols + block_cols - 1) / block_cols : 1;
@@ -184,7 +218,7 @@ int build_bounds(fg_spmm_plan *p) {
       n_blocks > 0 ? static_cast<double>(p->nnz) / (static_cast<double>(p->n_rows) * n_blocks) : 0.0;
   if (P == 1 || n_blocks < 2 || p->nnz == 0)
     n_blocks = 1;
-  else if (P == 0 && (cfg.spmm_blocked == 0 || (cfg.spmm_blocked < 0 && per_segment < 8.0)))
+  else if (P == 0 && (p->want_blocked == 0 || (p->want_blocked < 0 && per_segment < p->min_per_segment)))
     n_blocks = 1;
   p->force_blocks = P > 1;
   int *flag = nullptr;
@@ -250,6 +284,8 @@ int *config_slot(const char *key) {
   if (!strcmp(key, "sddmm.block_cols")) return &c.sddmm_block_cols;
   if (!strcmp(key, "sddmm.fast")) return &c.sddmm_fast;
   if (!strcmp(key, "sddmm.buffer_loads")) return &c.sddmm_buffer_loads;
+  if (!strcmp(key, "sddmm.rows")) return &c.sddmm_rows;
+  if (!strcmp(key, "sddmm.rows_blocks")) return &c.sddmm_rows_blocks;
   return nullptr;
 }
 
@@ -290,6 +326,14 @@ int fg_spmm_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32
 
 int fg_spmm_plan_create_partitioned(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr,
                                     const int32_t *indices, int32_t num_col_partitions, fg_spmm_plan **plan) {
+  return row_plan_create(n_rows, n_cols, nnz, indptr, indices, num_col_partitions, fg::config().spmm_block_cols,
+                         fg::config().spmm_blocked, 8.0, fg::config().spmm_sweep > 0, plan);
+}
+
+// want_block_cols / want_blocked / min_per_segment: see fg_spmm_plan; with_sweep: also build the column-sweep lists.
+static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr, const int32_t *indices,
+                           int32_t num_col_partitions, int32_t want_block_cols, int want_blocked,
+                           double min_per_segment, bool with_sweep, fg_spmm_plan **plan) {
   if (!plan) return fg::fail(FG_EINVAL, "plan output pointer is null");
   *plan = nullptr;
   if (num_col_partitions < 0)
@@ -338,6 +382,9 @@ int fg_spmm_plan_create_partitioned(int64_t n_rows, int64_t n_cols, int64_t nnz,
   p->row_order = nullptr;
   p->requested_partitions = num_col_partitions;
   p->force_blocks = false;
+  p->want_block_cols = want_block_cols;
+  p->want_blocked = want_blocked;
+  p->min_per_segment = min_per_segment;
   p->max_degree = max_degree;
   p->device = 0;
   hipError_t err = hipGetDevice(&p->device);
@@ -353,7 +400,7 @@ int fg_spmm_plan_create_partitioned(int64_t n_rows, int64_t n_cols, int64_t nnz,
   p->n_blocks = 0;
   p->block_cols = 0;
   int rc = build_bounds(p);
-  if (rc == FG_OK && p->n_blocks >= 2 && fg::config().spmm_sweep > 0)
+  if (rc == FG_OK && p->n_blocks >= 2 && with_sweep)
     rc = fg::sweep_build(host_indptr, order, p->seg, p->n_blocks, p->indices, p->nnz, &p->sweep);
   if (rc != FG_OK) {
     fg_spmm_plan_destroy(p);
@@ -423,6 +470,38 @@ int fg_sddmm_coo_mh_f32(int64_t nnz, const int32_t *row, const int32_t *col, con
   return fg::sddmm_launch(a, s, static_cast<hipStream_t>(stream));
 }
 
+// For a row-sorted edge list: rebuilds the row pointer and a row plan over (indptr, col) whose bounds table
+// cuts every row into column blocks (only when each row's column ids ascend; otherwise whole rows).
+// Leaves p->rows null for any other list.
+static int build_row_runs(fg_sddmm_plan *p, int32_t num_col_partitions) {
+  if (fg::config().sddmm_rows == 0 || p->nnz == 0 || p->n_rows >= 0x7fffffffLL || p->nnz > 0x7fffffffLL) return FG_OK;
+  int *flag = nullptr;
+  int bad = 0;
+  FG_HIP_TRY(hipMalloc(&flag, sizeof(int)));
+  hipError_t err = hipMemset(flag, 0, sizeof(int));
+  const unsigned grid = static_cast<unsigned>(std::min<int64_t>((p->nnz + 255) / 256, 16384));
+  if (err == hipSuccess) {
+    rows_sorted_kernel<<<dim3(grid), dim3(256)>>>(p->row, p->nnz, static_cast<int32_t>(p->n_rows), flag);
+    err = hipGetLastError();
+  }
+  if (err == hipSuccess) err = hipMemcpy(&bad, flag, sizeof(int), hipMemcpyDeviceToHost);
+  (void)hipFree(flag);
+  if (err != hipSuccess) return fg::fail(FG_EHIP, "row order check: %s", hipGetErrorString(err));
+  if (bad) return FG_OK;
+  err = hipMalloc(&p->indptr, sizeof(int32_t) * (p->n_rows + 1));
+  if (err != hipSuccess) {
+    p->indptr = nullptr;
+    return fg::fail(err == hipErrorOutOfMemory ? FG_ENOMEM : FG_EHIP, "row pointer: %s", hipGetErrorString(err));
+  }
+  indptr_from_rows_kernel<<<dim3(grid), dim3(256)>>>(p->row, p->nnz, static_cast<int32_t>(p->n_rows), p->indptr);
+  FG_HIP_TRY(hipGetLastError());
+  FG_HIP_TRY(hipDeviceSynchronize());
+  // same block width as the re-ordered edge list (sddmm_blocked.hip); a run costs a wave a fixed amount of
+  // work, so blocks need 8 edges per run on average (sparser lists keep whole rows and take the edge-list path)
+  return row_plan_create(p->n_rows, p->n_cols, p->nnz, p->indptr, p->col, num_col_partitions,
+                         fg::config().sddmm_block_cols, fg::config().sddmm_blocked, 8.0, false, &p->rows);
+}
+
 int fg_sddmm_plan_create(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,
                          fg_sddmm_plan **plan) {
   return fg_sddmm_plan_create_partitioned(nnz, n_rows, n_cols, row, col, 0, plan);
@@ -447,9 +526,17 @@ int fg_sddmm_plan_create_partitioned(int64_t nnz, int64_t n_rows, int64_t n_cols
   p->row = row;
   p->col = col;
   p->force_blocks = num_col_partitions > 1;
-  if (int rc = fg::sddmm_blocks_build(nnz, n_rows, n_cols, row, col, num_col_partitions, &p->blocks)) {
-    delete p;
+  if (int rc = build_row_runs(p, num_col_partitions)) {
+    fg_sddmm_plan_destroy(p);
     return rc;
+  }
+  // the re-ordered edge list serves the lists that the row-run kernel cannot take
+  const bool runs_blocked = p->rows && (p->rows->n_blocks >= 2 || num_col_partitions == 1);
+  if (!runs_blocked || fg::config().sddmm_rows == 0) {
+    if (int rc = fg::sddmm_blocks_build(nnz, n_rows, n_cols, row, col, num_col_partitions, &p->blocks)) {
+      fg_sddmm_plan_destroy(p);
+      return rc;
+    }
   }
   *plan = p;
   return FG_OK;
@@ -458,6 +545,8 @@ int fg_sddmm_plan_create_partitioned(int64_t nnz, int64_t n_rows, int64_t n_cols
 void fg_sddmm_plan_destroy(fg_sddmm_plan *plan) {
   if (!plan) return;
   fg::sddmm_blocks_free(&plan->blocks);
+  if (plan->rows) fg_spmm_plan_destroy(plan->rows);
+  if (plan->indptr) (void)hipFree(plan->indptr);
   delete plan;
 }
 
@@ -468,9 +557,39 @@ static bool sddmm_use_blocks(const fg_sddmm_plan *plan, const float *src, const 
          fg::aligned_to(dst, 16);
 }
 
+// Column blocks of the table that one pass of the row-run kernel takes together: the band of Src that a pass
+// gathers from (block width x tile bytes) should stay about one L2 (4 MB), so narrower tiles take wider
+// blocks.  Blocks that the caller sized (partition count, sddmm.block_cols) are used as they are.
+static int sddmm_rows_merge(const fg_sddmm_plan *plan, int32_t D) {
+  const fg_spmm_plan *r = plan->rows;
+  if (plan->force_blocks || r->want_block_cols > 0 || r->n_blocks < 2) return 1;
+  const int64_t band_cols = (int64_t{4} << 20) / (fg::sddmm_rows_tile(D) * 4);
+  return static_cast<int>(std::max<int64_t>(1, band_cols / r->block_cols));
+}
+
+static bool sddmm_use_row_runs(const fg_sddmm_plan *plan, const float *src, const float *dst, int32_t H, int32_t D) {
+  const int mode = fg::config().sddmm_rows;
+  if (!plan->rows || !plan->rows->seg || mode == 0) return false;
+  if (H != 1 || D % 4 != 0 || !fg::aligned_to(src, 16) || !fg::aligned_to(dst, 16)) return false;
+  if (mode > 0) return true;
+  if (plan->rows->n_blocks < 2) return false;  // whole rows: the edge-list kernels take it
+  if (plan->force_blocks) return true;
+  if (fg::config().sddmm_blocked == 0) return false;
+  return fg::config().sddmm_blocked > 0 || D >= 16;  // shorter rows leave most lanes of a 4-lane group idle
+}
+
 int fg_sddmm_coo_plan_f32(const fg_sddmm_plan *plan, const float *src, const float *dst, float *out, int32_t H,
                           int32_t D, void *stream) {
   if (!plan) return fg::fail(FG_EINVAL, "plan is null");
+  if (sddmm_use_row_runs(plan, src, dst, H, D)) {
+    if (int rc = check_heads(H, D)) return rc;
+    if (!src || !dst || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
+    const fg_spmm_plan *r = plan->rows;
+    return fg::sddmm_rows_launch(r->seg, r->row_order, static_cast<int32_t>(r->n_rows), r->n_blocks,
+                                 sddmm_rows_merge(plan, D), plan->col, src,
+                                 dst, out, plan->n_cols * int64_t{D} * 4, plan->n_rows * int64_t{D} * 4, D,
+                                 static_cast<hipStream_t>(stream));
+  }
   if (!sddmm_use_blocks(plan, src, dst, H, D)) {
     fg::SddmmArgs a;
     fg::SddmmShape s;
@@ -488,6 +607,19 @@ int fg_sddmm_plan_describe(const fg_sddmm_plan *plan, int32_t H, int32_t D, char
   if (!plan) return fg::fail(FG_EINVAL, "plan is null");
   if (!buf || cap <= 0) return fg::fail(FG_EINVAL, "no room for the description");
   alignas(16) static float dummy[4];
+  if (sddmm_use_row_runs(plan, dummy, dummy, H, D)) {
+    const int rows_tile = fg::sddmm_rows_tile(D);
+    const int merge = sddmm_rows_merge(plan, D);
+    snprintf(buf, static_cast<size_t>(cap),
+             "sddmm_coo nnz=%lld H=%d D=%d | kernel=row runs (row-sorted edge list), %d column blocks of %d, tile=%d "
+             "floats x %d tiles (one launch each), floats/lane=4 lanes/dot=%d | grid=(blocks, column blocks) x %d "
+             "threads each",
+             (long long)plan->nnz, H, D, (plan->rows->n_blocks + merge - 1) / merge,
+             static_cast<int>(std::min<int64_t>(int64_t{plan->rows->block_cols} * merge, 0x7fffffff)), rows_tile,
+             (D + rows_tile - 1) / rows_tile,
+             rows_tile / 4, fg::kBlockThreads);
+    return FG_OK;
+  }
   if (!sddmm_use_blocks(plan, dummy, dummy, H, D)) return fg_sddmm_describe(plan->nnz, H, D, buf, cap);
   const int64_t blocks = ((plan->nnz + 63) / 64 + fg::kWavesPerBlock - 1) / fg::kWavesPerBlock;
   snprintf(buf, static_cast<size_t>(cap),
@@ -528,7 +660,7 @@ int fg_config_set(const char *key, int32_t value) {
                     slot == &fg::config().spmm_blocked || slot == &fg::config().spmm_pipeline ||
                     slot == &fg::config().spmm_sweep || slot == &fg::config().sddmm_blocked ||
                     slot == &fg::config().spmm_buffer_loads || slot == &fg::config().sddmm_fast ||
-                    slot == &fg::config().sddmm_buffer_loads;
+                    slot == &fg::config().sddmm_buffer_loads || slot == &fg::config().sddmm_rows;
   // flags: 0 / 1 are explicit, anything negative restores the default;
   // sizes: 0 restores the default
   *slot = flag ? (value < 0 ? -1 : (value != 0)) : std::max(value, 0);

@@ -26,7 +26,7 @@ struct Config {
   int spmm_blocked = -1, spmm_block_cols = 0, spmm_pipeline = -1, spmm_pipe_blocks = 0;
   int spmm_sweep = -1, spmm_sweep_waves_per_cu = 0, spmm_buffer_loads = -1;
   int sddmm_group = 0, sddmm_batches = 0, sddmm_blocked = -1, sddmm_block_cols = 0;
-  int sddmm_fast = -1, sddmm_buffer_loads = -1;
+  int sddmm_fast = -1, sddmm_buffer_loads = -1, sddmm_rows = -1, sddmm_rows_blocks = 0;
 };
 Config &config();
 
@@ -137,6 +137,14 @@ int sddmm_blocked_launch(const SddmmBlocks &b, int64_t nnz, const float *src, co
 int sddmm_tile_launch(const int32_t *row_p, const int32_t *col_p, const int32_t *pos_p, int64_t nnz, const float *src,
                       const float *dst, float *out, int64_t src_bytes, int64_t dst_bytes, int32_t F, int tile,
                       hipStream_t stream);
+
+// Row-run kernel over (column block, row) runs of a row-sorted edge list: one launch per tile of
+// sddmm_rows_tile(F) floats, grid.y = column block.  seg / row_order are the bounds table and row list of a
+// row plan built on the same matrix; `merge` neighbouring blocks of the table are taken as one (sddmm.hip).
+int sddmm_rows_tile(int32_t F);
+int sddmm_rows_launch(const int32_t *seg, const int32_t *row_order, int32_t n_rows, int32_t n_blocks, int32_t merge,
+                      const int32_t *col, const float *src, const float *dst, float *out, int64_t src_bytes,
+                      int64_t dst_bytes, int32_t F, hipStream_t stream);
 
 inline bool aligned_to(const void *p, uintptr_t bytes) { return (reinterpret_cast<uintptr_t>(p) & (bytes - 1)) == 0; }
 

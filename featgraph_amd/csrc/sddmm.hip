@@ -13,6 +13,8 @@
 // Every output has a single writer and a fixed summation tree, so results are
 // deterministic and do not depend on the batch count; they do depend on G and
 // VEC, which are fixed functions of D and of the pointer alignment.
+#include <algorithm>
+
 #include "common.hpp"
 
 namespace fg {
@@ -214,6 +216,158 @@ int launch_fast_mode(const FastArgs &a, hipStream_t stream) {
   return FG_OK;
 }
 
+
+// ---------------------------------------------------------------------------
+// Row-run kernel for a row-sorted edge list (a COO list derived from CSR) with
+// column blocks.  A work item is one (column block, row) run of edges: they are
+// consecutive in the caller's list and share their Dst row, so the wave loads
+// that row's 64-float tile ONCE into registers (float4 per lane, the same in
+// each of its four 16-lane groups) and each edge then costs a single gathered
+// Src tile instead of two; the edge-list kernels above move 512 B per edge and
+// tile through L1, which is what bounds them once the gathers hit L2.  Items
+// are numbered block-major (blockIdx.y is the column block), so the resident
+// waves gather from one column block of Src at a time, as in the re-ordered
+// edge list, but results go straight to Out[e] with coalesced stores and no
+// re-ordered copy of the list exists.  Group g takes the edges lo + 4*round + g;
+// after at most 16 rounds a cross-lane move puts edge lo + l into lane l.
+// Like the SpMM pipelined kernel a wave keeps three items in flight: gathers of
+// item k, column ids / Dst tile / previous partial result of item k+1, bounds
+// of item k+2.
+struct RowsArgs {
+  const int32_t *seg;        // [(n_blocks + 1) * n_rows] run bounds, rows in visiting order
+  const int32_t *row_order;  // [n_rows]
+  const int32_t *col;        // the caller's column ids
+  const float *src;
+  const float *dst;
+  float *out;
+  int64_t src_bytes, dst_bytes;
+  int32_t n_rows, F;
+  int32_t first, valid;      // the tile this launch covers
+  int32_t n_blocks, merge;   // column blocks in the table; blockIdx.y covers `merge` neighbouring ones
+};
+
+// G: lanes per dot product (a tile is 4 * G floats); R: rounds whose gathers are issued together.
+template <bool ACC, bool BUF, int R, int G>
+__global__ __launch_bounds__(kBlockThreads) void sddmm_rows_kernel(const RowsArgs a) {
+  constexpr int NG = kWaveSize / G;  // edges per round
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int gl = lane & (G - 1);
+  const int g = lane / G;
+  const int n_waves = gridDim.x * kWavesPerBlock;
+  const int n = a.n_rows;
+  int item = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)));
+  const int32_t *const seg_lo = a.seg + static_cast<int64_t>(blockIdx.y) * a.merge * n;
+  const int32_t *const seg_hi = a.seg + static_cast<int64_t>(min((blockIdx.y + 1) * a.merge, a.n_blocks)) * n;
+  const VertexRows<BUF> src(a.src, a.src_bytes), dst(a.dst, a.dst_bytes);
+  const uint32_t row_bytes = static_cast<uint32_t>(a.F) * 4u;
+  const bool kok = gl * 4 < a.valid;
+  const uint32_t lane_bytes = static_cast<uint32_t>(a.first + (kok ? gl * 4 : a.valid - 4)) * 4u;
+  const int gather_from = G * (lane % NG) + lane / NG;  // lane holding the result of edge offset `lane`
+
+  auto bounds = [&](int it, int &lo, int &hi, int &row) {
+    lo = hi = row = 0;
+    if (it < n) {
+      lo = seg_lo[it];
+      hi = seg_hi[it];
+      row = a.row_order[it];
+    }
+  };
+  auto first_block = [&](int lo, int hi, int row, int &col, float4 &y, float &prev) {
+    col = 0;
+    prev = 0.0f;
+    y = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (hi > lo) {
+      if (lane < hi - lo) {
+        col = a.col[lo + lane];
+        if (ACC) prev = a.out[lo + lane];
+      }
+      y = dst.load(row, row_bytes, lane_bytes);
+    }
+  };
+
+  int lo_a, hi_a, row_a, col_a, lo_b, hi_b, row_b;
+  float4 y_a;
+  float prev_a;
+  bounds(item, lo_a, hi_a, row_a);
+  first_block(lo_a, hi_a, row_a, col_a, y_a, prev_a);
+  bounds(item + n_waves, lo_b, hi_b, row_b);
+
+  while (item < n) {
+    int lo_c, hi_c, row_c, col_b = 0;
+    float4 y_b = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    float prev_b = 0.0f;
+    bounds(item + 2 * n_waves, lo_c, hi_c, row_c);
+    bool next_asked = false;
+    auto ask_next = [&]() {
+      if (!next_asked) first_block(lo_b, hi_b, row_b, col_b, y_b, prev_b);
+      next_asked = true;
+    };
+
+    for (int e = lo_a; e < hi_a; e += kWaveSize) {
+      const int cnt = min(kWaveSize, hi_a - e);
+      int col_n = 0;
+      float prev_n = 0.0f;
+      const int rounds = (cnt + NG - 1) / NG;
+      float res = 0.0f;
+      // two batches of R rounds alternate: the gathers of one are in flight while the other is summed
+      float4 xa[R], xb[R];
+      auto issue = [&](int rb, float4(&x)[R]) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          // edges past the run's end read column id 0 of an idle lane: a valid row, result never stored
+          const int cc = __builtin_amdgcn_ds_bpermute(((NG * (rb + r) + g) & 63) << 2, col_a);
+          x[r] = src.load(cc, row_bytes, lane_bytes);
+        }
+      };
+      auto reduce = [&](int rb, const float4(&x)[R]) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          float p = 0.0f;
+          p = __builtin_fmaf(x[r].x, y_a.x, p);
+          p = __builtin_fmaf(x[r].y, y_a.y, p);
+          p = __builtin_fmaf(x[r].z, y_a.z, p);
+          p = __builtin_fmaf(x[r].w, y_a.w, p);
+          p = kok ? p : 0.0f;
+          p = group_sum<G>(p);
+          if (gl == rb + r) res = p;
+        }
+      };
+      issue(0, xa);
+      {  // behind this run's first gathers: the next run's operands and this run's next 64 ids
+        ask_next();
+        const int more = hi_a - (e + kWaveSize);
+        if (lane < more) {
+          col_n = a.col[e + kWaveSize + lane];
+          if (ACC) prev_n = a.out[e + kWaveSize + lane];
+        }
+      }
+      for (int rb = 0; rb < rounds; rb += 2 * R) {
+        const bool second = rb + R < rounds;
+        if (second) issue(rb + R, xb);
+        reduce(rb, xa);
+        if (rb + 2 * R < rounds) issue(rb + 2 * R, xa);
+        if (second) reduce(rb + R, xb);
+      }
+      const float mine = __int_as_float(__builtin_amdgcn_ds_bpermute(gather_from << 2, __float_as_int(res)));
+      if (lane < cnt) a.out[e + lane] = ACC ? prev_a + mine : mine;
+      col_a = col_n;
+      prev_a = prev_n;
+    }
+    ask_next();
+
+    lo_a = lo_b;
+    hi_a = hi_b;
+    row_a = row_b;
+    col_a = col_b;
+    y_a = y_b;
+    prev_a = prev_b;
+    lo_b = lo_c;
+    hi_b = hi_c;
+    row_b = row_c;
+    item += n_waves;
+  }
+}
+
 template <int VEC, int G>
 int launch(const SddmmArgs &a, hipStream_t stream) {
   const int64_t per_wave = static_cast<int64_t>(a.batches) * kWaveSize;
@@ -307,6 +461,63 @@ int sddmm_tile_launch(const int32_t *row_p, const int32_t *col_p, const int32_t 
   f.first = tile * 64;
   f.valid = F - tile * 64 < 64 ? F - tile * 64 : 64;
   return tile == 0 ? launch_fast_mode<16, 1, false, 1>(f, stream) : launch_fast_mode<16, 1, false, 2>(f, stream);
+}
+
+template <int G>
+static void rows_dispatch(const RowsArgs &a, bool acc, bool buf, dim3 grid, hipStream_t stream) {
+  if (!acc) {
+    if (buf)
+      sddmm_rows_kernel<false, true, 2, G><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+    else
+      sddmm_rows_kernel<false, false, 2, G><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+  } else {
+    if (buf)
+      sddmm_rows_kernel<true, true, 2, G><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+    else
+      sddmm_rows_kernel<true, false, 2, G><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+  }
+}
+
+int sddmm_rows_tile(int32_t F) { return F <= 16 ? 16 : F <= 32 ? 32 : 64; }
+
+int sddmm_rows_launch(const int32_t *seg, const int32_t *row_order, int32_t n_rows, int32_t n_blocks, int32_t merge,
+                      const int32_t *col, const float *src, const float *dst, float *out, int64_t src_bytes,
+                      int64_t dst_bytes, int32_t F, hipStream_t stream) {
+  if (n_rows == 0) return FG_OK;
+  RowsArgs a;
+  a.seg = seg;
+  a.row_order = row_order;
+  a.col = col;
+  a.src = src;
+  a.dst = dst;
+  a.out = out;
+  a.src_bytes = src_bytes;
+  a.dst_bytes = dst_bytes;
+  a.n_rows = n_rows;
+  a.F = F;
+  int64_t blocks = config().sddmm_rows_blocks > 0 ? config().sddmm_rows_blocks : 16384;
+  blocks = std::max<int64_t>(1, std::min<int64_t>(blocks, (n_rows + kWavesPerBlock - 1) / kWavesPerBlock));
+  merge = std::max(1, std::min(merge, n_blocks));
+  a.n_blocks = n_blocks;
+  a.merge = merge;
+  const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>((n_blocks + merge - 1) / merge));
+  const bool buf = src_bytes < (int64_t{1} << 32) && dst_bytes < (int64_t{1} << 32) && config().sddmm_buffer_loads != 0;
+  // tile width: 64 floats, or the whole row when it is shorter (then fewer lanes share a dot product)
+  const int tile = sddmm_rows_tile(F);
+  const int G = tile / 4;
+  const int n_tiles = (F + tile - 1) / tile;
+  for (int t = 0; t < n_tiles; ++t) {
+    a.first = t * tile;
+    a.valid = std::min(F - t * tile, tile);
+    if (G == 4)
+      rows_dispatch<4>(a, t > 0, buf, grid, stream);
+    else if (G == 8)
+      rows_dispatch<8>(a, t > 0, buf, grid, stream);
+    else
+      rows_dispatch<16>(a, t > 0, buf, grid, stream);
+    FG_HIP_TRY(hipGetLastError());
+  }
+  return FG_OK;
 }
 
 int sddmm_launch(const SddmmArgs &a, const SddmmShape &s, hipStream_t stream) {

@@ -31,7 +31,8 @@ def config_guard():
     _lib.config_set("sddmm.group", 0)
     _lib.config_set("sddmm.batches", 0)
     _lib.config_set("sddmm.block_cols", 0)
-    for key in ("sddmm.blocked", "sddmm.fast", "sddmm.buffer_loads"):
+    _lib.config_set("sddmm.rows_blocks", 0)
+    for key in ("sddmm.blocked", "sddmm.fast", "sddmm.buffer_loads", "sddmm.rows"):
         _lib.config_set(key, -1)
 
 
@@ -133,6 +134,7 @@ def test_column_blocked_edge_list(config_guard, F):
     src, dst = datasets.sddmm_operands(coo, F)
     want = ref.sddmm_x86(coo.row, coo.col, src, dst)
     exact = ref.sddmm_f64(coo.row, coo.col, src, dst)
+    _lib.config_set("sddmm.rows", 0)                                 # this graph's list is row-sorted: keep it off the row-run kernel
     _lib.config_set("sddmm.blocked", 0)
     plain = _run_sddmm(coo, src, dst)
     outs = []
@@ -141,7 +143,7 @@ def test_column_blocked_edge_list(config_guard, F):
         _lib.config_set("sddmm.block_cols", block_cols)
         module = VanillaSDDMMhip(coo)
         text = module.lower_to_ir([placeholder(src.shape), placeholder(dst.shape)], {}, {})
-        assert "column blocks of %d" % block_cols in text
+        assert "column-blocked edge list" in text and "column blocks of %d" % block_cols in text
         module.build([placeholder(src.shape), placeholder(dst.shape)], {}, {})
         module.out_tvm.tensor.fill_(7.0)                             # stale contents must not leak into the sums
         out = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
@@ -200,6 +202,90 @@ def test_unrolled_kernel_against_the_general_one(config_guard, shape):
     assert np.array_equal(outs[(1, 0)], outs[(1, 1)])               # addressing mode cannot change a bit
     if D <= 64:
         assert np.array_equal(outs[(0, 0)], outs[(1, 0)])           # one step per lane: same summation tree
+
+
+# ---------------------------------------------------------------- row runs of a row-sorted edge list
+def _describe(module, src, dst):
+    return module.lower_to_ir([placeholder(src.shape), placeholder(dst.shape)], {}, {})
+
+
+@pytest.mark.parametrize("F", [4, 32, 64, 68, 100, 128, 260, 512])
+def test_row_runs_of_a_row_sorted_list(config_guard, F):
+    coo = datasets.config_graph("c2-mini").tocoo()                   # derived from CSR: rows ascend, columns ascend within a row
+    src, dst = datasets.sddmm_operands(coo, F)
+    want = ref.sddmm_x86(coo.row, coo.col, src, dst)
+    exact = ref.sddmm_f64(coo.row, coo.col, src, dst)
+    _lib.config_set("sddmm.blocked", 1)
+    outs = []
+    for block_cols, grid in ((64, 0), (1000, 0), (1000, 3)):
+        _lib.config_set("sddmm.block_cols", block_cols)
+        _lib.config_set("sddmm.rows_blocks", grid)                   # 3 workgroups: every wave walks many runs
+        module = VanillaSDDMMhip(coo)
+        text = _describe(module, src, dst)
+        assert "row runs" in text and "column blocks of %d" % block_cols in text
+        module.build([placeholder(src.shape), placeholder(dst.shape)], {}, {})
+        module.out_tvm.tensor.fill_(7.0)                             # stale contents must not leak into the sums
+        out = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
+        np.testing.assert_allclose(out, want, rtol=RTOL, atol=ATOL)
+        np.testing.assert_allclose(out, exact, rtol=RTOL, atol=ATOL)
+        outs.append(out)
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[1], outs[2])
+    _lib.config_set("sddmm.rows", 0)                                 # same tiles, same summation tree as the re-ordered list
+    module = VanillaSDDMMhip(coo)
+    assert "column-blocked edge list" in _describe(module, src, dst)
+    assert np.array_equal(_run_sddmm(coo, src, dst), outs[0])
+
+
+def test_row_runs_only_for_row_sorted_lists(config_guard):
+    _lib.config_set("sddmm.blocked", 1)
+    _lib.config_set("sddmm.block_cols", 500)
+    coo = datasets.config_graph("c2-mini").tocoo()
+    src, dst = datasets.sddmm_operands(coo, 64)
+    assert "row runs" in _describe(VanillaSDDMMhip(coo), src, dst)
+    rng = np.random.default_rng(9)
+    perm = rng.permutation(coo.nnz)
+    shuffled = scipy.sparse.coo_matrix((coo.data[perm], (coo.row[perm], coo.col[perm])), shape=coo.shape)
+    assert "column-blocked edge list" in _describe(VanillaSDDMMhip(shuffled), src, dst)
+    # rows ascend but the columns inside a row do not: runs of one column block are no longer contiguous
+    order = np.lexsort((rng.random(coo.nnz), coo.row))
+    ragged = scipy.sparse.coo_matrix((coo.data[order], (coo.row[order], coo.col[order])), shape=coo.shape)
+    assert np.all(np.diff(ragged.row) >= 0) and np.any(np.diff(ragged.col)[np.diff(ragged.row) == 0] < 0)
+    assert "column-blocked edge list" in _describe(VanillaSDDMMhip(ragged), src, dst)
+    base = _run_sddmm(coo, src, dst)
+    inv = np.empty_like(order)
+    inv[order] = np.arange(coo.nnz)
+    assert np.array_equal(_run_sddmm(ragged, src, dst)[inv], base)
+    # 30 floats or several heads: neither blocked kernel applies
+    src30, dst30 = datasets.sddmm_operands(coo, 30)
+    assert "row runs" not in _describe(VanillaSDDMMhip(coo), src30, dst30)
+
+
+def test_row_runs_on_awkward_structures(config_guard):
+    _lib.config_set("sddmm.blocked", 1)
+    _lib.config_set("sddmm.block_cols", 128)
+    rng = np.random.default_rng(10)
+    n_rows, n_cols = 70, 700
+    dense = np.zeros((n_rows, n_cols), dtype=bool)
+    dense[5] = True                                                  # 128 edges in every block: runs longer than a wave
+    dense[6, :130] = True                                            # 128 + 2
+    dense[7, 127:129] = True                                         # one edge on each side of a block border
+    dense[20:40] = rng.random((20, n_cols)) < 0.03
+    dense[69, 699] = True                                            # rows 0-4, 8-19 and 40-68 stay empty
+    csr = scipy.sparse.csr_matrix(dense.astype(np.float32))
+    coo = csr.tocoo()
+    dup = scipy.sparse.coo_matrix((np.ones(2 * coo.nnz, np.float32), (np.repeat(coo.row, 2), np.repeat(coo.col, 2))),
+                                  shape=coo.shape)                   # every edge twice, still sorted
+    for F in (64, 96, 200):
+        src = rng.integers(-8, 9, (n_cols, F)).astype(np.float32)
+        dst = rng.integers(-8, 9, (n_rows, F)).astype(np.float32)
+        for adj in (coo, dup):
+            module = VanillaSDDMMhip(adj)
+            assert "row runs" in _describe(module, src, dst)
+            want = (src[adj.col].astype(np.int64) * dst[adj.row].astype(np.int64)).sum(-1).astype(np.float32)
+            assert np.array_equal(_run_sddmm(adj, src, dst), want)   # exact on integers
+    one = scipy.sparse.coo_matrix((np.ones(1, np.float32), ([69], [3])), shape=(n_rows, n_cols))
+    src, dst = datasets.sddmm_operands(one, 64)
+    np.testing.assert_allclose(_run_sddmm(one, src, dst), ref.sddmm_f64(one.row, one.col, src, dst), rtol=RTOL, atol=ATOL)
 
 
 # the reference's partitioned x86 test (tests/test_module_sddmm.py:16-41), partition arguments included
