@@ -55,6 +55,10 @@ struct fg_spmm_plan {
   int want_blocked;
   double min_per_segment;
   fg::SweepPlan sweep;  // per-wave block-major lists (optional)
+  // Records of the several-rows-per-wave kernel: whole rows, and column-block passes for its tiles of 16, 32
+  // and 64 floats (tables with the same blocks-per-pass share their records).
+  fg::MultiRuns multi_whole;
+  fg::MultiRuns multi_tile[3];
 };
 
 struct fg_sddmm_plan {
@@ -71,7 +75,7 @@ struct fg_sddmm_plan {
 
 static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr, const int32_t *indices,
                            int32_t num_col_partitions, int32_t want_block_cols, int want_blocked,
-                           double min_per_segment, bool with_sweep, fg_spmm_plan **plan);
+                           double min_per_segment, bool with_sweep, bool with_multi, fg_spmm_plan **plan);
 
 namespace {
 
@@ -180,6 +184,99 @@ bool use_column_blocks(const fg_spmm_plan *plan, const fg::SpmmArgs &a, const fg
   return band_bytes > (int64_t{6} << 20);
 }
 
+int multi_tile_index(int tile) { return tile == 16 ? 0 : tile == 32 ? 1 : 2; }
+
+// Column blocks of the plan's table that one pass of the several-rows-per-wave kernel takes together, for
+// tiles of `tile` floats: the band of the feature matrix that a pass gathers from (block width x tile bytes)
+// should stay about one L2 (4 MB), so narrower tiles take wider blocks; blocks that the caller sized
+// (partition count, spmm.block_cols) are used as they are.
+int multi_merge(const fg_spmm_plan *plan, int tile) {
+  if (plan->n_blocks < 2) return 1;
+  if (plan->force_blocks || plan->want_block_cols > 0) return 1;
+  const int64_t m = (int64_t{4} << 20) / (tile * 4) / std::max(plan->block_cols, 1);
+  return static_cast<int>(std::min<int64_t>(std::max<int64_t>(m, 1), plan->n_blocks));
+}
+
+int multi_build(fg_spmm_plan *p) {
+  if (fg::config().spmm_multi == 0 || !p->seg || !p->row_order || p->n_rows == 0) return FG_OK;
+  const int32_t n = static_cast<int32_t>(p->n_rows);
+  if (int rc = fg::multi_runs_build(p->seg, p->row_order, n, p->n_blocks, p->n_blocks, &p->multi_whole)) return rc;
+  if (p->n_blocks < 2) return FG_OK;
+  const int tiles[3] = {16, 32, 64};
+  for (int t = 0; t < 3; ++t) {
+    const int merge = multi_merge(p, tiles[t]);
+    if (merge >= p->n_blocks) continue;  // one pass: the whole-row records
+    bool shared = false;
+    for (int u = 0; u < t && !shared; ++u)
+      if (p->multi_tile[u].rec && p->multi_tile[u].merge == merge) {
+        p->multi_tile[t] = p->multi_tile[u];
+        shared = true;
+      }
+    if (!shared)
+      if (int rc = fg::multi_runs_build(p->seg, p->row_order, n, p->n_blocks, merge, &p->multi_tile[t])) return rc;
+  }
+  return FG_OK;
+}
+
+void multi_free(fg_spmm_plan *p) {
+  for (int t = 0; t < 3; ++t) {
+    for (int u = t + 1; u < 3; ++u)
+      if (p->multi_tile[u].rec && p->multi_tile[u].rec == p->multi_tile[t].rec) p->multi_tile[u] = fg::MultiRuns();
+    fg::multi_runs_free(&p->multi_tile[t]);
+  }
+  fg::multi_runs_free(&p->multi_whole);
+}
+
+// The records that a call uses: null when the kernel does not take the call.  The kernel is the default
+// wherever it applies; an explicit launch shape (tuning keys, the caller's feature tiling) asks for the
+// row-slot / wave-per-row kernels.
+const fg::MultiRuns *multi_table(const fg_spmm_plan *plan, const fg::SpmmArgs &a, int32_t feat_tiles) {
+  const fg::Config &c = fg::config();
+  if (c.spmm_multi == 0 || !fg::spmm_multi_applies(a) || !plan->multi_whole.rec) return nullptr;
+  if (c.spmm_multi < 0 && !(feat_tiles == 0 && c.spmm_vec == 0 && c.spmm_lpr == 0 && c.spmm_unroll == 0 &&
+                            c.spmm_pipeline < 0 && c.spmm_scalar_path < 0 && c.spmm_sorted != 0))
+    return nullptr;
+  const int tile = fg::spmm_multi_tile(a.F);
+  const fg::MultiRuns *blocked = &plan->multi_tile[multi_tile_index(tile)];
+  if (!blocked->rec || blocked->passes < 2) return &plan->multi_whole;
+  if (plan->force_blocks) return blocked;
+  if (c.spmm_blocked == 0) return &plan->multi_whole;
+  const int64_t band_bytes = static_cast<int64_t>(plan->n_cols) * std::min<int>(tile, a.F) * 4;
+  if (c.spmm_blocked < 0 && band_bytes <= (int64_t{6} << 20)) return &plan->multi_whole;  // fits an L2 anyway
+  return blocked;
+}
+
+int multi_run(const fg_spmm_plan *plan, const fg::MultiRuns *runs, fg::SpmmArgs a, hipStream_t st) {
+  const int tile = fg::spmm_multi_tile(a.F);
+  const int n_tiles = (a.F + tile - 1) / tile;
+  const int64_t n = plan->n_rows;
+  auto long_split = [&](int pass) {
+    a.long_runs = runs->long_runs[pass];
+    a.long_blocks = std::min((a.long_runs + fg::kWavesPerBlock - 1) / fg::kWavesPerBlock, 2048);
+  };
+  if (runs->passes == 1) {
+    a.runs = runs->rec;
+    long_split(0);
+    a.tile_base = 0;
+    a.n_tiles = n_tiles;
+    a.accumulate = 0;
+    return fg::spmm_multi_launch(a, st);
+  }
+  // one launch per (tile, pass), passes in ascending column order: launches on a stream run one after the
+  // other, so every row's sum still grows in CSR order, carried from pass to pass in `out`
+  a.n_tiles = 1;
+  for (int t = 0; t < n_tiles; ++t) {
+    a.tile_base = t;
+    for (int b = 0; b < runs->passes; ++b) {
+      a.runs = runs->rec + static_cast<int64_t>(b) * n;
+      long_split(b);
+      a.accumulate = b > 0;
+      if (int rc = fg::spmm_multi_launch(a, st)) return rc;
+    }
+  }
+  return FG_OK;
+}
+
 // n_rows / n_cols: matrix extents when known (a plan knows them), else 0.
 int sddmm_prepare(int64_t nnz, const int32_t *row, const int32_t *col, const float *src, const float *dst,
                   float *out, int32_t H, int32_t D, fg::SddmmArgs *a, fg::SddmmShape *s, int64_t n_rows = 0,
@@ -278,6 +375,9 @@ int *config_slot(const char *key) {
   if (!strcmp(key, "spmm.buffer_loads")) return &c.spmm_buffer_loads;
   if (!strcmp(key, "spmm.sweep_waves_per_cu")) return &c.spmm_sweep_waves_per_cu;
   if (!strcmp(key, "spmm.pipe_blocks")) return &c.spmm_pipe_blocks;
+  if (!strcmp(key, "spmm.multi")) return &c.spmm_multi;
+  if (!strcmp(key, "spmm.multi_blocks")) return &c.spmm_multi_blocks;
+  if (!strcmp(key, "spmm.multi_long")) return &c.spmm_multi_long;
   if (!strcmp(key, "sddmm.group")) return &c.sddmm_group;
   if (!strcmp(key, "sddmm.batches")) return &c.sddmm_batches;
   if (!strcmp(key, "sddmm.blocked")) return &c.sddmm_blocked;
@@ -327,13 +427,14 @@ int fg_spmm_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32
 int fg_spmm_plan_create_partitioned(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr,
                                     const int32_t *indices, int32_t num_col_partitions, fg_spmm_plan **plan) {
   return row_plan_create(n_rows, n_cols, nnz, indptr, indices, num_col_partitions, fg::config().spmm_block_cols,
-                         fg::config().spmm_blocked, 8.0, fg::config().spmm_sweep > 0, plan);
+                         fg::config().spmm_blocked, 8.0, fg::config().spmm_sweep > 0, true, plan);
 }
 
-// want_block_cols / want_blocked / min_per_segment: see fg_spmm_plan; with_sweep: also build the column-sweep lists.
+// want_block_cols / want_blocked / min_per_segment: see fg_spmm_plan; with_sweep / with_multi: also build the
+// column-sweep lists / the records of the several-rows-per-wave kernel.
 static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr, const int32_t *indices,
                            int32_t num_col_partitions, int32_t want_block_cols, int want_blocked,
-                           double min_per_segment, bool with_sweep, fg_spmm_plan **plan) {
+                           double min_per_segment, bool with_sweep, bool with_multi, fg_spmm_plan **plan) {
   if (!plan) return fg::fail(FG_EINVAL, "plan output pointer is null");
   *plan = nullptr;
   if (num_col_partitions < 0)
@@ -400,6 +501,7 @@ static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const in
   p->n_blocks = 0;
   p->block_cols = 0;
   int rc = build_bounds(p);
+  if (rc == FG_OK && with_multi) rc = multi_build(p);
   if (rc == FG_OK && p->n_blocks >= 2 && with_sweep)
     rc = fg::sweep_build(host_indptr, order, p->seg, p->n_blocks, p->indices, p->nnz, &p->sweep);
   if (rc != FG_OK) {
@@ -415,6 +517,7 @@ void fg_spmm_plan_destroy(fg_spmm_plan *plan) {
   if (plan->row_order) (void)hipFree(plan->row_order);
   if (plan->seg) (void)hipFree(plan->seg);
   fg::sweep_free(&plan->sweep);
+  multi_free(plan);
   delete plan;
 }
 
@@ -438,6 +541,7 @@ int fg_spmm_csr_mh_f32(const fg_spmm_plan *plan, const float *feat, const float 
   if (int rc = spmm_prepare(plan, feat, w, out, H, D, feat_tiles, &a, &s)) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (use_sweep(plan, a)) return fg::sweep_launch(plan->sweep, a, fg::config().spmm_unroll, st);
+  if (const fg::MultiRuns *runs = multi_table(plan, a, feat_tiles)) return multi_run(plan, runs, a, st);
   if (!use_column_blocks(plan, a, s)) return fg::spmm_launch(a, s, st);
   // One launch per (feature tile, column block), blocks in ascending column
   // order: launches on one stream run one after the other, so every row's sum
@@ -499,7 +603,7 @@ static int build_row_runs(fg_sddmm_plan *p, int32_t num_col_partitions) {
   // same block width as the re-ordered edge list (sddmm_blocked.hip); a run costs a wave a fixed amount of
   // work, so blocks need 8 edges per run on average (sparser lists keep whole rows and take the edge-list path)
   return row_plan_create(p->n_rows, p->n_cols, p->nnz, p->indptr, p->col, num_col_partitions,
-                         fg::config().sddmm_block_cols, fg::config().sddmm_blocked, 8.0, false, &p->rows);
+                         fg::config().sddmm_block_cols, fg::config().sddmm_blocked, 8.0, false, false, &p->rows);
 }
 
 int fg_sddmm_plan_create(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,
@@ -660,7 +764,8 @@ int fg_config_set(const char *key, int32_t value) {
                     slot == &fg::config().spmm_blocked || slot == &fg::config().spmm_pipeline ||
                     slot == &fg::config().spmm_sweep || slot == &fg::config().sddmm_blocked ||
                     slot == &fg::config().spmm_buffer_loads || slot == &fg::config().sddmm_fast ||
-                    slot == &fg::config().sddmm_buffer_loads || slot == &fg::config().sddmm_rows;
+                    slot == &fg::config().sddmm_buffer_loads || slot == &fg::config().sddmm_rows ||
+                    slot == &fg::config().spmm_multi;
   // flags: 0 / 1 are explicit, anything negative restores the default;
   // sizes: 0 restores the default
   *slot = flag ? (value < 0 ? -1 : (value != 0)) : std::max(value, 0);
@@ -691,6 +796,22 @@ int fg_spmm_describe(const fg_spmm_plan *plan, int32_t H, int32_t D, int32_t fea
              (a.F + 63) / 64, plan->n_blocks, plan->block_cols, sp.waves, sp.rows_per_wave, (long long)sp.mean_load,
              (long long)sp.max_load, sp.generations, sp.waves / fg::kWavesPerBlock, (a.F + 63) / 64,
              fg::kBlockThreads);
+    return FG_OK;
+  }
+  if (const fg::MultiRuns *runs = multi_table(plan, a, feat_tiles)) {
+    const int tile = fg::spmm_multi_tile(a.F);
+    const int n_tiles = (a.F + tile - 1) / tile;
+    const int n_passes = runs->passes, merge = runs->merge;
+    char passes[112] = "1 launch";
+    if (n_passes > 1)
+      snprintf(passes, sizeof(passes), "%d launches (%d tiles x %d column blocks of %d)", n_tiles * n_passes, n_tiles,
+               n_passes, static_cast<int>(std::min<int64_t>(int64_t{plan->block_cols} * merge, 0x7fffffff)));
+    snprintf(buf, static_cast<size_t>(cap),
+             "spmm_csr rows=%lld cols=%lld nnz=%lld max_degree=%d H=%d D=%d | kernel=rows-per-wave(pipelined) "
+             "floats/lane=4 lanes/row=%d rows/wave=%d tile=%d floats x %d tiles gathers-in-flight=%d "
+             "rows=by-descending-degree | %s",
+             (long long)plan->n_rows, (long long)plan->n_cols, (long long)plan->nnz, plan->max_degree, H, D, tile / 4,
+             fg::kWaveSize / (tile / 4), tile, n_tiles, tile / 4, passes);
     return FG_OK;
   }
   const int rows_per_wave = fg::kWaveSize / s.lpr;

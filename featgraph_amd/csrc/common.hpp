@@ -25,6 +25,7 @@ struct Config {
   int spmm_vec = 0, spmm_lpr = 0, spmm_unroll = 0, spmm_scalar_path = -1, spmm_sorted = -1;
   int spmm_blocked = -1, spmm_block_cols = 0, spmm_pipeline = -1, spmm_pipe_blocks = 0;
   int spmm_sweep = -1, spmm_sweep_waves_per_cu = 0, spmm_buffer_loads = -1;
+  int spmm_multi = -1, spmm_multi_blocks = 0, spmm_multi_long = 0;
   int sddmm_group = 0, sddmm_batches = 0, sddmm_blocked = -1, sddmm_block_cols = 0;
   int sddmm_fast = -1, sddmm_buffer_loads = -1, sddmm_rows = -1, sddmm_rows_blocks = 0;
 };
@@ -58,6 +59,10 @@ struct SpmmArgs {
   const int32_t *seg_hi = nullptr;
   int32_t tile_base = 0;
   int32_t accumulate = 0;
+  // several-rows-per-wave kernel: one pass's records {first nonzero, one past the last, row id, 0}, n_rows of them
+  const int4 *runs = nullptr;
+  int32_t long_runs = 0;    // the first long_runs records are long runs: one wave each, in the first
+  int32_t long_blocks = 0;  // long_blocks workgroups of the grid
 };
 
 struct SpmmShape {
@@ -91,6 +96,21 @@ int sweep_build(const std::vector<int32_t> &indptr, const std::vector<int32_t> &
 void sweep_free(SweepPlan *sp);
 int sweep_launch(const SweepPlan &sp, const SpmmArgs &a, int unroll, hipStream_t stream);
 int spmm_launch(const SpmmArgs &a, const SpmmShape &s, hipStream_t stream);
+
+// Several-rows-per-wave kernel with 16-byte gathers (spmm_multi.hip): single head, feature length a multiple
+// of 4, 16-byte aligned operands, rows and bounds from the plan.  Tiles are spmm_multi_tile(F) floats wide.
+struct MultiRuns {
+  int4 *rec = nullptr;  // [passes * n_rows], device, owned by the plan
+  int32_t merge = 0;    // column blocks of the bounds table per pass
+  int32_t passes = 0;
+  int32_t *long_runs = nullptr;  // [passes], host, owned: how many of a pass's records are long runs
+};
+int multi_runs_build(const int32_t *seg, const int32_t *row_order, int32_t n_rows, int32_t n_blocks, int32_t merge,
+                     MultiRuns *out);
+void multi_runs_free(MultiRuns *r);
+int spmm_multi_tile(int32_t F);
+bool spmm_multi_applies(const SpmmArgs &a);
+int spmm_multi_launch(const SpmmArgs &a, hipStream_t stream);
 
 // One launch of the edge-parallel SDDMM kernel over n_ve = nnz * H dot
 // products of length D ("virtual edges": edge e, head h -> e * H + h).

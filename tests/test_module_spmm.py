@@ -36,10 +36,10 @@ def _oracle(adj, feat_np, P=1):
 def config_guard():
     yield
     for key in ("spmm.vec", "spmm.lpr", "spmm.unroll", "spmm.block_cols", "spmm.pipe_blocks",
-                "spmm.sweep_waves_per_cu"):
+                "spmm.sweep_waves_per_cu", "spmm.multi_blocks", "spmm.multi_long"):
         _lib.config_set(key, 0)
     for key in ("spmm.scalar_path", "spmm.sorted", "spmm.blocked", "spmm.pipeline", "spmm.sweep",
-                "spmm.buffer_loads"):
+                "spmm.buffer_loads", "spmm.multi"):
         _lib.config_set(key, -1)
 
 
@@ -288,6 +288,82 @@ def test_index_check_entry_point():
     n_bad = ctypes.c_int64(-1)
     _lib.check(_lib.lib().fg_check_indices(idx.numel(), idx.data_ptr(), 10, ctypes.byref(n_bad), None))
     assert n_bad.value == 2
+
+
+# ---------------------------------------------------------------- several rows per wave, 16-byte gathers
+def _describe(module, feat):
+    return module.lower_to_ir([placeholder(feat.shape)], {}, {})
+
+
+@pytest.mark.parametrize("blocks", [(0, 0), (1, 7), (1, 100), (1, 1500)])
+@pytest.mark.parametrize("long_run", [0, 8, 1 << 20])
+def test_rows_per_wave_kernel_gives_the_same_bits(config_guard, blocks, long_run):
+    adj = datasets.config_graph("c2-mini")
+    _lib.config_set("spmm.blocked", blocks[0])
+    _lib.config_set("spmm.block_cols", blocks[1])
+    _lib.config_set("spmm.multi_long", long_run)       # 8: nearly every run takes the one-wave-per-run path; 2^20: none
+    module = VanillaSpMMhip(adj)
+    for F in (4, 8, 16, 20, 32, 36, 64, 68, 200, 512):
+        feat = datasets.spmm_operands(adj, F)
+        text = _describe(module, feat)
+        assert "rows-per-wave" in text and (("column blocks of %d" % blocks[1]) in text) == bool(blocks[0])
+        module.build([placeholder(feat.shape)], {}, {})
+        module.out_tvm.tensor.fill_(3.0)               # stale contents must not leak into the carried sums
+        out = module.run([nd.array(feat, module.ctx)]).asnumpy()
+        assert np.array_equal(out, _oracle(adj, feat)), "F=%d" % F
+
+
+def test_rows_per_wave_kernel_only_where_it_applies(config_guard, adj_127x255):
+    module = VanillaSpMMhip(adj_127x255)
+    assert "rows-per-wave" in _describe(module, np.empty((255, 64), np.float32))
+    assert "rows-per-wave" not in _describe(module, np.empty((255, 30), np.float32))       # not a multiple of 4 floats
+    assert "rows-per-wave" not in module.lower_to_ir([placeholder((255, 64))], {"num_feat_partitions": 2}, {})
+    _lib.config_set("spmm.lpr", 64)                    # an explicit launch shape asks for the other kernels
+    assert "rows-per-wave" not in _describe(module, np.empty((255, 64), np.float32))
+    _lib.config_set("spmm.lpr", 0)
+    _lib.config_set("spmm.multi", 0)
+    assert "rows-per-wave" not in _describe(module, np.empty((255, 64), np.float32))
+    feat = datasets.spmm_operands(adj_127x255, 64)
+    off = _run_spmm(adj_127x255, feat)
+    _lib.config_set("spmm.multi", -1)
+    assert np.array_equal(_run_spmm(adj_127x255, feat), off)
+
+
+@pytest.mark.parametrize("long_run", [0, 16, 300])
+def test_rows_per_wave_kernel_on_degenerate_rows(config_guard, long_run):
+    _lib.config_set("spmm.multi_long", long_run)
+    rng = np.random.default_rng(21)
+    # rows of length 0, 1, 63, 64, 65, 129, 255..257 and two long ones; fewer rows than one wave's groups at 16 floats
+    lens = np.array([0, 1, 63, 0, 64, 65, 129, 0, 0, 1000, 2, 0, 255, 256, 257, 2100], dtype=np.int64)
+    indptr = np.zeros(len(lens) + 1, dtype=np.int32)
+    np.cumsum(lens, out=indptr[1:])
+    indices = np.concatenate([np.sort(rng.integers(0, 500, l)) for l in lens]).astype(np.int32)
+    vals = rng.random(indptr[-1], dtype=np.float32)
+    adj = scipy.sparse.csr_matrix((vals, indices, indptr), shape=(len(lens), 500))
+    for blocked, block_cols, grid, buf in ((0, 0, 0, -1), (1, 64, 0, -1), (1, 64, 1, 0), (0, 0, 1, 0)):
+        _lib.config_set("spmm.blocked", blocked)
+        _lib.config_set("spmm.block_cols", block_cols)
+        _lib.config_set("spmm.multi_blocks", grid)     # one workgroup: every wave walks several items
+        _lib.config_set("spmm.buffer_loads", buf)
+        module = VanillaSpMMhip(adj)
+        for F in (12, 32, 70 * 4):
+            feat = rng.standard_normal((500, F), dtype=np.float32)
+            assert "rows-per-wave" in _describe(module, feat)
+            module.build([placeholder(feat.shape)], {}, {})
+            module.out_tvm.tensor.fill_(9.0)
+            out = module.run([nd.array(feat, module.ctx)]).asnumpy()
+            assert np.array_equal(out, ref.spmm_csr_x86(indptr, indices, vals, feat)), (blocked, grid, F)
+
+
+def test_rows_per_wave_kernel_with_the_callers_partitions(adj_127x255):
+    feat = datasets.spmm_operands(adj_127x255, 64)
+    want = _oracle(adj_127x255, feat)
+    for P in (1, 2, 7):
+        module = VanillaSpMMhip(adj_127x255, P)
+        text = _describe(module, feat)
+        assert "rows-per-wave" in text and (("%d column blocks" % P) in text) == (P > 1)
+        module.build([placeholder(feat.shape)], {}, {})
+        assert np.array_equal(module.run([nd.array(feat, module.ctx)]).asnumpy(), want)
 
 
 # ---------------------------------------------------------------- column-blocked passes
