@@ -12,7 +12,8 @@
  * Conventions
  *   - Every data pointer is DEVICE memory owned by the caller.  The library
  *     never copies user data between host and device and never allocates or
- *     frees a caller-visible buffer.  A plan owns only its private row list.
+ *     frees a caller-visible buffer.  A plan owns only its private schedule
+ *     arrays (row list, bounds, run records; sizes are given with each plan).
  *   - Index arrays are int32, values and features float32, row-major, dense.
  *   - Kernels are enqueued on `stream` (a hipStream_t passed as void*, NULL =
  *     the default stream) and the call returns without synchronising.
@@ -58,9 +59,12 @@ FG_API const char *fg_last_error(void);
  * by ascending row id).  When the matrix is wide and dense enough for column
  * blocking to pay off and every row's column ids ascend, it also stores, per
  * block of 16384 columns, where that block starts inside every row (one device
- * pass over indices; (n_cols/16384 + 2) * n_rows int32).  The plan BORROWS
- * indptr and indices: both must stay alive and unchanged until
- * fg_spmm_plan_destroy.
+ * pass over indices; (n_cols/16384 + 2) * n_rows int32), and for the default
+ * kernel one 16-byte record {first nonzero, one past the last, row id} per row
+ * and column-block pass, each pass sorted by descending run length (device
+ * radix sorts; with blocks about (n_cols/16384) * 2 * n_rows records, else
+ * n_rows).  The plan BORROWS indptr and indices: both must stay alive and
+ * unchanged until fg_spmm_plan_destroy.
  */
 FG_API int fg_spmm_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr,
                         const int32_t *indices, fg_spmm_plan **plan);
@@ -114,11 +118,14 @@ FG_API int fg_sddmm_coo_f32(int64_t nnz, const int32_t *row, const int32_t *col,
 
 /*
  * Cache-blocking schedule for one COO edge list; takes the place that
- * SDDMMbase.__init__ gives to 2-D graph partitioning (module/sddmm.py:45-49):
- * when the matrix is wide and dense enough, stores the edge list re-ordered by
- * blocks of 16384 columns (stable, so each block keeps the caller's order)
- * together with every edge's original position: 12 bytes per edge of device
- * memory, built with one device radix sort.  Results are always written in the
+ * SDDMMbase.__init__ gives to 2-D graph partitioning (module/sddmm.py:45-49).
+ * When the matrix is wide and dense enough: for a list whose row ids ascend
+ * and whose column ids ascend inside every row (COO derived from CSR) it
+ * rebuilds the row pointer and stores where every block of 16384 columns
+ * starts inside every row ((n_cols/16384 + 3) * n_rows int32); for any other
+ * list it stores the edge list re-ordered by blocks of 16384 columns (stable,
+ * so each block keeps the caller's order) together with every edge's original
+ * position: 12 bytes per edge, one device radix sort.  Results are always written in the
  * caller's edge order; there is no edge_mapping to apply.  The plan BORROWS row
  * and col, which must stay alive and unchanged until fg_sddmm_plan_destroy.
  */
@@ -134,9 +141,11 @@ FG_API void fg_sddmm_plan_destroy(fg_sddmm_plan *plan);
 /*
  * fg_sddmm_coo_mh_f32 on the plan's edge list.  With H = 1, F a multiple of 4
  * and 16-byte aligned operands a blocked plan runs one launch per 64-float
- * feature tile over the re-ordered list (each tile adds its partial dot
- * product to Out, the reference's feature tiling: op/vanilla_sddmm.py:49-60);
- * otherwise this is the plain kernel.  Both agree within float32 rounding.
+ * feature tile (each tile adds its partial dot product to Out, the reference's
+ * feature tiling: op/vanilla_sddmm.py:49-60): over (row, column block) runs of
+ * a row-sorted list, one Dst tile held in registers per run, or over the
+ * re-ordered list; otherwise this is the plain kernel.  All agree within
+ * float32 rounding.
  */
 FG_API int fg_sddmm_coo_plan_f32(const fg_sddmm_plan *plan, const float *src, const float *dst, float *out, int32_t H,
                                  int32_t D, void *stream);
@@ -172,10 +181,18 @@ FG_API int fg_check_indices(int64_t n, const int32_t *idx, int64_t bound, int64_
  * "spmm.sweep" (1: also build, and use, the per-wave block-major lists of the
  * experimental column-sweep kernel; read at plan creation and at launch),
  * "spmm.sweep_waves_per_cu" (its resident waves per CU),
+ * "spmm.multi" (0/1: never / always use the several-rows-per-wave kernel where
+ * it applies; by default it runs unless one of the shape keys above is set;
+ * read at plan creation and at launch), "spmm.multi_blocks" (its grid size),
+ * "spmm.multi_long" (run length from which a run gets a wave of its own,
+ * default 512; read at plan creation),
  * "sddmm.blocked" (0/1: never / always build and use column blocks, read at
  * plan creation), "sddmm.block_cols" (columns per block, read at plan creation),
  * "sddmm.group" (lanes per dot product: 1..16),
- * "sddmm.batches" (64-edge batches per wave).  Value 0 restores the default of
+ * "sddmm.batches" (64-edge batches per wave), "sddmm.fast" (0/1: unrolled
+ * kernel for D in 16..512), "sddmm.buffer_loads" (0/1), "sddmm.rows" (0/1:
+ * never / always use the row-run kernel when the plan has a row plan; read at
+ * plan creation and at launch), "sddmm.rows_blocks" (its grid size).  Value 0 restores the default of
  * a size; for the 0/1 flags a negative value does.
  * The spmm.* keys change the launch shape only; "sddmm.group" also changes the
  * shape of the summation tree, i.e. the last bits of an SDDMM result.
