@@ -355,3 +355,30 @@ def test_each_head_is_a_vanilla_sddmm_on_its_slice():
     for h in (0, 5):
         one = _run_sddmm(coo, np.ascontiguousarray(src[:, h]), np.ascontiguousarray(dst[:, h]))
         assert np.array_equal(mh[:, h], one)
+
+
+# ---------------------------------------------------------------- seeded random structures, default kernel choice
+@pytest.mark.parametrize("seed", range(10))
+def test_random_structures_under_random_schedules(config_guard, seed):
+    rng = np.random.default_rng(2000 + seed)
+    n_rows, n_cols = int(rng.integers(1, 400)), int(rng.integers(1, 3000))
+    dens = float(rng.choice([0.002, 0.02, 0.2]))
+    mask = rng.random((n_rows, n_cols)) < dens
+    mask[rng.integers(0, n_rows, 2)] |= rng.random((2, n_cols)) < 0.8          # two long rows
+    coo = scipy.sparse.csr_matrix(mask.astype(np.float32)).tocoo()
+    if rng.random() < 0.3:                                                     # not row-sorted: the edge-list path
+        perm = rng.permutation(coo.nnz)
+        coo = scipy.sparse.coo_matrix((coo.data[perm], (coo.row[perm], coo.col[perm])), shape=coo.shape)
+    _lib.config_set("sddmm.blocked", int(rng.integers(0, 2)))
+    _lib.config_set("sddmm.block_cols", int(rng.choice([1, 5, 64, 300, 1 << 20])))
+    _lib.config_set("sddmm.rows_blocks", int(rng.choice([0, 1, 2])))
+    module = VanillaSDDMMhip(coo)
+    for F in rng.choice([1, 3, 4, 8, 12, 16, 24, 32, 48, 64, 100, 128, 192, 260], 5, replace=False):
+        F = int(F)
+        src = rng.integers(-8, 9, (n_cols, F)).astype(np.float32)
+        dst = rng.integers(-8, 9, (n_rows, F)).astype(np.float32)
+        module.build([placeholder(src.shape), placeholder(dst.shape)], {}, {})
+        module.out_tvm.tensor.fill_(-1.0)
+        out = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
+        want = (src[coo.col].astype(np.int64) * dst[coo.row].astype(np.int64)).sum(-1).astype(np.float32)
+        assert np.array_equal(out, want), (seed, F)                            # exact on integers

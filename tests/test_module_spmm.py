@@ -530,3 +530,33 @@ def test_multihead_launch_shapes_give_the_same_bits(config_guard, key, values):
             _lib.config_set("spmm.lpr", 64)
         _lib.config_set(key, v)
         assert np.array_equal(_run_mh(adj, feat, w), want), "%s=%d" % (key, v)
+
+
+# ---------------------------------------------------------------- seeded random structures, default kernel choice
+def _random_csr(rng, n_rows, n_cols, mean_deg, hubs):
+    deg = np.minimum(rng.poisson(mean_deg, n_rows), n_cols)
+    deg[rng.integers(0, n_rows, hubs)] = np.minimum(rng.integers(n_cols // 2, n_cols + 1, hubs), n_cols)
+    deg[rng.random(n_rows) < 0.15] = 0
+    indptr = np.zeros(n_rows + 1, dtype=np.int32)
+    np.cumsum(deg, out=indptr[1:])
+    indices = np.concatenate([np.sort(rng.choice(n_cols, d, replace=False)) for d in deg] + [np.empty(0, np.int64)])
+    vals = rng.standard_normal(int(indptr[-1])).astype(np.float32)
+    return scipy.sparse.csr_matrix((vals, indices.astype(np.int32), indptr), shape=(n_rows, n_cols))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_structures_bit_exact_under_random_schedules(config_guard, seed):
+    rng = np.random.default_rng(1000 + seed)
+    n_rows, n_cols = int(rng.integers(1, 400)), int(rng.integers(1, 3000))
+    adj = _random_csr(rng, n_rows, n_cols, float(rng.choice([0.5, 3, 20, 90])), int(rng.integers(0, 4)))
+    _lib.config_set("spmm.blocked", int(rng.integers(0, 2)))
+    _lib.config_set("spmm.block_cols", int(rng.choice([1, 5, 64, 300, 1 << 20])))
+    _lib.config_set("spmm.multi_long", int(rng.choice([0, 4, 64, 700])))
+    _lib.config_set("spmm.multi_blocks", int(rng.choice([0, 1, 2])))
+    module = VanillaSpMMhip(adj)
+    for F in rng.choice([1, 3, 4, 8, 12, 16, 24, 32, 48, 64, 100, 128, 192, 260], 5, replace=False):
+        feat = rng.standard_normal((n_cols, int(F))).astype(np.float32)
+        module.build([placeholder(feat.shape)], {}, {})
+        module.out_tvm.tensor.fill_(-1.0)
+        out = module.run([nd.array(feat, module.ctx)]).asnumpy()
+        assert np.array_equal(out, ref.spmm_csr_x86(adj.indptr, adj.indices, adj.data, feat)), (seed, int(F))
