@@ -67,8 +67,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--feat-len", type=int, default=64, help="feature length of the timed step")
     ap.add_argument("--graph", default="c2", help="named synthetic configuration (featgraph_amd.datasets.CONFIGS)")
-    ap.add_argument("--only", choices=["all", "spmm", "sddmm", "copy"], default="all",
-                    help="spmm / sddmm / copy: run just that kernel (for profiler runs), no sweep, no CPU leg")
+    ap.add_argument("--only", choices=["all", "spmm", "sddmm", "copy", "mh_sddmm", "mh_spmm"], default="all",
+                    help="spmm / sddmm / copy: run just that kernel (for profiler runs), no sweep, no CPU leg; "
+                         "mh_sddmm / mh_spmm: the multi-head operators (8 heads of --feat-len floats, use --graph c4)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="skip the feature-length sweep")
     args = ap.parse_args()
@@ -79,7 +80,7 @@ def main():
     import numpy as np
     import torch
     from featgraph_amd import _lib, datasets, nd, placeholder
-    from featgraph_amd.module import VanillaSDDMMhip, VanillaSpMMhip
+    from featgraph_amd.module import MultiHeadSDDMMhip, MultiHeadSpMMhip, VanillaSDDMMhip, VanillaSpMMhip
 
     _lib.lib()  # fail now if the HIP library is missing
     if not torch.cuda.is_available():
@@ -117,6 +118,27 @@ def main():
         time.time() - t))
     F = args.feat_len
     out = {}
+
+    if args.only in ("mh_sddmm", "mh_spmm"):
+        # per-head forms of the two operators: [N, H, D] features, [nnz, H] edge weights / results
+        H, D = 8, F
+        if args.only == "mh_sddmm":
+            op = MultiHeadSDDMMhip(adj.tocoo())
+            ins = [nd.array(torch.randn((n_cols, H, D), dtype=torch.float32, device=dev)),
+                   nd.array(torch.randn((n_rows, H, D), dtype=torch.float32, device=dev))]
+            op.build([placeholder((n_cols, H, D)), placeholder((n_rows, H, D))], {}, {})
+            b = nnz * (8 + 8 * H * D + 4 * H)
+        else:
+            op = MultiHeadSpMMhip(adj)
+            ins = [nd.array(torch.randn((n_cols, H, D), dtype=torch.float32, device=dev)),
+                   nd.array(torch.rand((nnz, H), dtype=torch.float32, device=dev))]
+            op.build([placeholder((n_cols, H, D)), placeholder((nnz, H))], {}, {})
+            b = nnz * (4 + 4 * H + 4 * H * D) + n_rows * (4 + 4 * H * D)
+        ms = timed(lambda: op.run(ins), args.steps, args.warmup)
+        print(json.dumps({"kernel": args.only, "graph": args.graph, "H": H, "D": D, "ms": ms,
+                          "GFLOPs": 2.0 * nnz * H * D / ms / 1e6, "algorithmic_bytes": b, "alg_GBps": b / ms / 1e6,
+                          "frac": b / ms / 1e6 / HBM_PEAK_GBPS}))
+        return
 
     spmm = sddmm = None
     if args.only in ("all", "spmm"):
