@@ -530,18 +530,23 @@ SpmmShape spmm_choose_shape(const SpmmArgs &a, int feat_tiles) {
   // 256 MB Infinity Cache (the 2.45M-vertex multi-head graph: 627 MB): then
   // every gather goes to HBM whatever the tiling, and wider tiles win by
   // reading the index and weight streams fewer times.
-  if (static_cast<int64_t>(a.n_cols) * 256 > (int64_t{192} << 20)) want = a.F < 128 ? a.F : 128;
+  const bool beyond_cache = static_cast<int64_t>(a.n_cols) * 256 > (int64_t{192} << 20);
+  if (beyond_cache) want = a.F < 128 ? a.F : 128;
   if (feat_tiles >= 1) want = (a.F + feat_tiles - 1) / feat_tiles;
   int vec = 1;
   while (vec < max_vec && (want + vec - 1) / vec > kWaveSize) vec *= 2;
+  // ... and there two rows per wave with 16-byte gathers measured best (2.45M-vertex graph, 8 heads of 64
+  // floats: 23.5 ms against 25.6 ms for a wave per row with 8-byte gathers)
+  const bool two_rows = beyond_cache && feat_tiles < 1 && want == 128 && max_vec == 4;
+  if (two_rows) vec = 4;
   s.vec = (cfg.spmm_vec > 0 && cfg.spmm_vec <= max_vec) ? cfg.spmm_vec : vec;
   int lanes = pow2_ceil((want + s.vec - 1) / s.vec);
   if (lanes < 8) lanes = 8;
   // a wave per row with idle lanes (pipelined kernel) beats two rows per wave at 17..63 floats
-  if (lanes > 16 && feat_tiles < 1) lanes = kWaveSize;
+  if (lanes > 16 && feat_tiles < 1 && !two_rows) lanes = kWaveSize;
   if (lanes > kWaveSize) lanes = kWaveSize;
   s.lpr = cfg.spmm_lpr > 0 ? cfg.spmm_lpr : lanes;
-  s.unroll = cfg.spmm_unroll > 0 ? cfg.spmm_unroll : (s.lpr == 32 ? 32 : (s.lpr >= 16 ? 16 : 8));
+  s.unroll = cfg.spmm_unroll > 0 ? cfg.spmm_unroll : (two_rows ? 4 : s.lpr == 32 ? 32 : (s.lpr >= 16 ? 16 : 8));
   s.scalar_path = cfg.spmm_scalar_path >= 0 ? cfg.spmm_scalar_path : 1;
   if (s.lpr != kWaveSize) s.scalar_path = 0;
   s.pipeline = cfg.spmm_pipeline >= 0 ? cfg.spmm_pipeline : 1;
