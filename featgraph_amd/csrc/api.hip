@@ -206,6 +206,10 @@ int multi_build(fg_spmm_plan *p) {
   for (int t = 0; t < 3; ++t) {
     const int merge = multi_merge(p, tiles[t]);
     if (merge >= p->n_blocks) continue;  // one pass: the whole-row records
+    // 16 bytes per row and pass: with very many passes (a caller's large partition count on a thin matrix) the
+    // records would dwarf the matrix itself; such plans keep the bounds table and the wave-per-row kernels
+    const int64_t passes = (p->n_blocks + merge - 1) / merge;
+    if (passes * p->n_rows * 16 > std::max<int64_t>(4 * p->nnz * 8, int64_t{256} << 20)) continue;
     bool shared = false;
     for (int u = 0; u < t && !shared; ++u)
       if (p->multi_tile[u].rec && p->multi_tile[u].merge == merge) {
@@ -238,8 +242,9 @@ const fg::MultiRuns *multi_table(const fg_spmm_plan *plan, const fg::SpmmArgs &a
     return nullptr;
   const int tile = fg::spmm_multi_tile(a.F);
   const fg::MultiRuns *blocked = &plan->multi_tile[multi_tile_index(tile)];
+  if (plan->force_blocks && plan->n_blocks >= 2)  // the caller's blocks: the kernels that have them
+    return blocked->rec && blocked->passes >= 2 ? blocked : nullptr;
   if (!blocked->rec || blocked->passes < 2) return &plan->multi_whole;
-  if (plan->force_blocks) return blocked;
   if (c.spmm_blocked == 0) return &plan->multi_whole;
   const int64_t band_bytes = static_cast<int64_t>(plan->n_cols) * std::min<int>(tile, a.F) * 4;
   if (c.spmm_blocked < 0 && band_bytes <= (int64_t{6} << 20)) return &plan->multi_whole;  // fits an L2 anyway

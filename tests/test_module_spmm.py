@@ -366,6 +366,22 @@ def test_rows_per_wave_kernel_with_the_callers_partitions(adj_127x255):
         assert np.array_equal(module.run([nd.array(feat, module.ctx)]).asnumpy(), want)
 
 
+def test_very_many_partitions_keep_the_bounds_table_only(config_guard):
+    # 16 bytes per row and pass would be 324 MB of records for a 36 KB matrix: the plan skips them and the
+    # wave-per-row kernels run the caller's 4500 blocks
+    rng = np.random.default_rng(41)
+    n = 4500
+    adj = scipy.sparse.random(n, n, density=1.0 / n, format="csr", dtype=np.float32, random_state=rng)
+    adj.sort_indices()
+    feat = rng.standard_normal((n, 8)).astype(np.float32)
+    module = VanillaSpMMhip(adj, n)
+    text = _describe(module, feat)
+    assert "rows-per-wave" not in text and "%d column blocks" % n in text
+    module.build([placeholder(feat.shape)], {}, {})
+    out = module.run([nd.array(feat, module.ctx)]).asnumpy()
+    assert np.array_equal(out, _oracle(adj, feat))
+
+
 # ---------------------------------------------------------------- column-blocked passes
 @pytest.mark.parametrize("block_cols", [7, 100, 1500])
 @pytest.mark.parametrize("shape", [(4, 16, 0), (1, 64, 1), (1, 64, 0), (2, 32, 0), (1, 32, 0), (1, 64, 2), (2, 64, 2)])
