@@ -235,10 +235,10 @@ def main():
         from oracle import ref
         cores = ref.num_threads()
         work = np.empty((n_cols + n_rows) * F, dtype=np.float32)
-        runs = 3
         t0 = time.time()
         cpu_out = ref.spmm_csr_x86(adj.indptr, adj.indices, adj.data, feat_np, 1, work)   # warm-up, kept for parity
         first = time.time() - t0
+        runs = int(max(1, min(20, 10.0 / max(first, 1e-3))))   # about ten seconds of CPU work
         if first > 10.0:
             runs, cpu_s = 1, first
         else:
