@@ -97,6 +97,27 @@ FG_API int fg_spmm_csr_f32(const fg_spmm_plan *plan, const float *feat, const fl
                     int32_t feat_tiles, void *stream);
 
 /*
+ * fg_spmm_csr_f32 without a plan and without any allocation.  No counterpart in
+ * the reference: it is for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc) and therefore cannot call fg_spmm_plan_create.  The row schedule
+ * that a plan keeps in allocated memory (rows by descending degree and their
+ * bounds) is rebuilt on the device at every call, by degree class, inside a
+ * fixed 12 MiB array that is part of the library image, one copy per GPU;
+ * the SpMM kernels of fg_spmm_csr_f32 then run over it.  Same result bits as
+ * fg_spmm_csr_f32.  Limits: n_rows <= 1048576 (FG_EUNSUPPORTED beyond).  The
+ * call enqueues kernels on `stream` and returns; it calls no hipMalloc /
+ * hipFree, copies nothing and never synchronises.  Every call on a GPU uses
+ * that GPU's one array: calls that overlap in time on the same GPU (two
+ * streams, two threads) race on it and must be serialised by the caller.
+ * indptr CONTENTS are the caller's contract (non-decreasing, 0 .. nnz); rows
+ * whose bounds are out of range come out as zeros.
+ */
+FG_API int fg_spmm_csr_noalloc_f32(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr,
+                                   const int32_t *indices, const float *vals, const float *feat, float *out,
+                                   int32_t F, void *stream);
+
+/*
  * Multi-head generalised SpMM (no counterpart in the reference, whose
  * op/__init__.py:1-5 exports vanilla operators only; same message function as
  * op/vanilla_spmm.py:46-53 with a per-head weight):
