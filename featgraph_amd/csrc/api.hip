@@ -54,7 +54,6 @@ struct fg_spmm_plan {
   int32_t want_block_cols;
   int want_blocked;
   double min_per_segment;
-  fg::SweepPlan sweep;  // per-wave block-major lists (optional)
   // Records of the several-rows-per-wave kernel: whole rows, and column-block passes for its tiles of 16, 32
   // and 64 floats (tables with the same blocks-per-pass share their records).
   fg::MultiRuns multi_whole;
@@ -66,6 +65,7 @@ struct fg_sddmm_plan {
   const int32_t *row;  // borrowed, device
   const int32_t *col;  // borrowed, device
   bool force_blocks;   // the caller asked for column partitions: use them at every feature length
+  int device = 0;      // the device that was current at creation
   fg::SddmmBlocks blocks;
   // Row-sorted lists (a COO list derived from CSR): the row pointer rebuilt from `row`, and a row plan over
   // it (visiting order + per-column-block bounds) for the row-run kernel.  Null otherwise.
@@ -75,7 +75,7 @@ struct fg_sddmm_plan {
 
 static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr, const int32_t *indices,
                            int32_t num_col_partitions, int32_t want_block_cols, int want_blocked,
-                           double min_per_segment, bool with_sweep, bool with_multi, fg_spmm_plan **plan);
+                           double min_per_segment, bool with_multi, fg_spmm_plan **plan);
 
 namespace {
 
@@ -132,6 +132,16 @@ __global__ void indptr_from_rows_kernel(const int32_t *row, int64_t nnz, int32_t
   }
 }
 
+// A plan's arrays live on the device that was current when it was built; launching with another device
+// current would hand kernels on that device pointers into this one's memory.
+int check_device(int plan_device) {
+  int now = -1;
+  FG_HIP_TRY(hipGetDevice(&now));
+  if (now != plan_device)
+    return fg::fail(FG_EINVAL, "the plan was built on device %d but device %d is current", plan_device, now);
+  return FG_OK;
+}
+
 int check_heads(int32_t H, int32_t D) {
   if (H < 1 || D < 1) return fg::fail(FG_EINVAL, "H = %d and D = %d must both be positive", H, D);
   if (static_cast<int64_t>(H) * D > (1 << 20))
@@ -143,6 +153,7 @@ int spmm_prepare(const fg_spmm_plan *plan, const float *feat, const float *w, fl
                  int32_t feat_tiles, fg::SpmmArgs *a, fg::SpmmShape *s) {
   if (!plan) return fg::fail(FG_EINVAL, "plan is null");
   if (int rc = check_heads(H, D)) return rc;
+  if (int rc = check_device(plan->device)) return rc;
   if (feat_tiles < 0) return fg::fail(FG_EINVAL, "feat_tiles = %d is negative", feat_tiles);
   if (plan->n_rows > 0 && !out) return fg::fail(FG_EINVAL, "out is null");
   if (plan->nnz > 0 && (!feat || !w)) return fg::fail(FG_EINVAL, "feat or edge values are null");
@@ -165,12 +176,6 @@ int spmm_prepare(const fg_spmm_plan *plan, const float *feat, const float *w, fl
   a->n_tiles = (a->F + s->tile_width() - 1) / s->tile_width();
   a->n_slots = static_cast<int64_t>(a->n_tiles) * a->n_rows;
   return FG_OK;
-}
-
-bool use_sweep(const fg_spmm_plan *plan, const fg::SpmmArgs &a) {
-  // built and used only on request: on the 232,965-vertex benchmark graph it runs 3.0 ms at 64 floats
-  // against 2.4 ms for the per-block launches (its waves drift apart: 61 % L2 hits against 73 %)
-  return plan->sweep.generations != 0 && fg::config().spmm_sweep > 0 && a.H * a.D >= 1;
 }
 
 bool use_column_blocks(const fg_spmm_plan *plan, const fg::SpmmArgs &a, const fg::SpmmShape &s) {
@@ -376,9 +381,7 @@ int *config_slot(const char *key) {
   if (!strcmp(key, "spmm.blocked")) return &c.spmm_blocked;
   if (!strcmp(key, "spmm.block_cols")) return &c.spmm_block_cols;
   if (!strcmp(key, "spmm.pipeline")) return &c.spmm_pipeline;
-  if (!strcmp(key, "spmm.sweep")) return &c.spmm_sweep;
   if (!strcmp(key, "spmm.buffer_loads")) return &c.spmm_buffer_loads;
-  if (!strcmp(key, "spmm.sweep_waves_per_cu")) return &c.spmm_sweep_waves_per_cu;
   if (!strcmp(key, "spmm.pipe_blocks")) return &c.spmm_pipe_blocks;
   if (!strcmp(key, "spmm.multi")) return &c.spmm_multi;
   if (!strcmp(key, "spmm.multi_blocks")) return &c.spmm_multi_blocks;
@@ -432,14 +435,14 @@ int fg_spmm_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32
 int fg_spmm_plan_create_partitioned(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr,
                                     const int32_t *indices, int32_t num_col_partitions, fg_spmm_plan **plan) {
   return row_plan_create(n_rows, n_cols, nnz, indptr, indices, num_col_partitions, fg::config().spmm_block_cols,
-                         fg::config().spmm_blocked, 8.0, fg::config().spmm_sweep > 0, true, plan);
+                         fg::config().spmm_blocked, 8.0, true, plan);
 }
 
-// want_block_cols / want_blocked / min_per_segment: see fg_spmm_plan; with_sweep / with_multi: also build the
-// column-sweep lists / the records of the several-rows-per-wave kernel.
+// want_block_cols / want_blocked / min_per_segment: see fg_spmm_plan; with_multi: also build the records of the
+// several-rows-per-wave kernel.
 static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr, const int32_t *indices,
                            int32_t num_col_partitions, int32_t want_block_cols, int want_blocked,
-                           double min_per_segment, bool with_sweep, bool with_multi, fg_spmm_plan **plan) {
+                           double min_per_segment, bool with_multi, fg_spmm_plan **plan) {
   if (!plan) return fg::fail(FG_EINVAL, "plan output pointer is null");
   *plan = nullptr;
   if (num_col_partitions < 0)
@@ -507,8 +510,6 @@ static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const in
   p->block_cols = 0;
   int rc = build_bounds(p);
   if (rc == FG_OK && with_multi) rc = multi_build(p);
-  if (rc == FG_OK && p->n_blocks >= 2 && with_sweep)
-    rc = fg::sweep_build(host_indptr, order, p->seg, p->n_blocks, p->indices, p->nnz, &p->sweep);
   if (rc != FG_OK) {
     fg_spmm_plan_destroy(p);
     return rc;
@@ -521,7 +522,6 @@ void fg_spmm_plan_destroy(fg_spmm_plan *plan) {
   if (!plan) return;
   if (plan->row_order) (void)hipFree(plan->row_order);
   if (plan->seg) (void)hipFree(plan->seg);
-  fg::sweep_free(&plan->sweep);
   multi_free(plan);
   delete plan;
 }
@@ -545,7 +545,6 @@ int fg_spmm_csr_mh_f32(const fg_spmm_plan *plan, const float *feat, const float 
   fg::SpmmShape s;
   if (int rc = spmm_prepare(plan, feat, w, out, H, D, feat_tiles, &a, &s)) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (use_sweep(plan, a)) return fg::sweep_launch(plan->sweep, a, fg::config().spmm_unroll, st);
   if (const fg::MultiRuns *runs = multi_table(plan, a, feat_tiles)) return multi_run(plan, runs, a, st);
   if (!use_column_blocks(plan, a, s)) return fg::spmm_launch(a, s, st);
   // One launch per (feature tile, column block), blocks in ascending column
@@ -608,7 +607,7 @@ static int build_row_runs(fg_sddmm_plan *p, int32_t num_col_partitions) {
   // same block width as the re-ordered edge list (sddmm_blocked.hip); a run costs a wave a fixed amount of
   // work, so blocks need 8 edges per run on average (sparser lists keep whole rows and take the edge-list path)
   return row_plan_create(p->n_rows, p->n_cols, p->nnz, p->indptr, p->col, num_col_partitions,
-                         fg::config().sddmm_block_cols, fg::config().sddmm_blocked, 8.0, false, false, &p->rows);
+                         fg::config().sddmm_block_cols, fg::config().sddmm_blocked, 8.0, false, &p->rows);
 }
 
 int fg_sddmm_plan_create(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,
@@ -635,6 +634,10 @@ int fg_sddmm_plan_create_partitioned(int64_t nnz, int64_t n_rows, int64_t n_cols
   p->row = row;
   p->col = col;
   p->force_blocks = num_col_partitions > 1;
+  if (hipGetDevice(&p->device) != hipSuccess) {
+    delete p;
+    return fg::fail(FG_EHIP, "hipGetDevice failed");
+  }
   if (int rc = build_row_runs(p, num_col_partitions)) {
     fg_sddmm_plan_destroy(p);
     return rc;
@@ -690,6 +693,8 @@ static bool sddmm_use_row_runs(const fg_sddmm_plan *plan, const float *src, cons
 int fg_sddmm_coo_plan_f32(const fg_sddmm_plan *plan, const float *src, const float *dst, float *out, int32_t H,
                           int32_t D, void *stream) {
   if (!plan) return fg::fail(FG_EINVAL, "plan is null");
+  if (plan->nnz > 0)
+    if (int rc = check_device(plan->device)) return rc;
   if (sddmm_use_row_runs(plan, src, dst, H, D)) {
     if (int rc = check_heads(H, D)) return rc;
     if (!src || !dst || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
@@ -767,7 +772,7 @@ int fg_config_set(const char *key, int32_t value) {
   if (!slot) return fg::fail(FG_EINVAL, "unknown configuration key '%s'", key ? key : "(null)");
   const bool flag = slot == &fg::config().spmm_scalar_path || slot == &fg::config().spmm_sorted ||
                     slot == &fg::config().spmm_blocked || slot == &fg::config().spmm_pipeline ||
-                    slot == &fg::config().spmm_sweep || slot == &fg::config().sddmm_blocked ||
+                    slot == &fg::config().sddmm_blocked ||
                     slot == &fg::config().spmm_buffer_loads || slot == &fg::config().sddmm_fast ||
                     slot == &fg::config().sddmm_buffer_loads || slot == &fg::config().sddmm_rows ||
                     slot == &fg::config().spmm_multi;
@@ -791,18 +796,6 @@ int fg_spmm_describe(const fg_spmm_plan *plan, int32_t H, int32_t D, int32_t fea
   // shape selection looks at pointer alignment only; describe the aligned case
   alignas(16) static float dummy[4];
   if (int rc = spmm_prepare(plan, dummy, dummy, dummy, H, D, feat_tiles, &a, &s)) return rc;
-  if (use_sweep(plan, a)) {
-    const fg::SweepPlan &sp = plan->sweep;
-    snprintf(buf, static_cast<size_t>(cap),
-             "spmm_csr rows=%lld cols=%lld nnz=%lld max_degree=%d H=%d D=%d | kernel=column-sweep tile=64 floats x %d "
-             "tiles, %d column blocks of %d, %d resident waves x %d rows each, nonzeros per wave mean %lld max %lld | "
-             "%d launch(es), grid=%d x %d blocks x %d threads each",
-             (long long)plan->n_rows, (long long)plan->n_cols, (long long)plan->nnz, plan->max_degree, H, D,
-             (a.F + 63) / 64, plan->n_blocks, plan->block_cols, sp.waves, sp.rows_per_wave, (long long)sp.mean_load,
-             (long long)sp.max_load, sp.generations, sp.waves / fg::kWavesPerBlock, (a.F + 63) / 64,
-             fg::kBlockThreads);
-    return FG_OK;
-  }
   if (const fg::MultiRuns *runs = multi_table(plan, a, feat_tiles)) {
     const int tile = fg::spmm_multi_tile(a.F);
     const int n_tiles = (a.F + tile - 1) / tile;

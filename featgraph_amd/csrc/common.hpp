@@ -24,7 +24,7 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 struct Config {
   int spmm_vec = 0, spmm_lpr = 0, spmm_unroll = 0, spmm_scalar_path = -1, spmm_sorted = -1;
   int spmm_blocked = -1, spmm_block_cols = 0, spmm_pipeline = -1, spmm_pipe_blocks = 0;
-  int spmm_sweep = -1, spmm_sweep_waves_per_cu = 0, spmm_buffer_loads = -1;
+  int spmm_buffer_loads = -1;
   int spmm_multi = -1, spmm_multi_blocks = 0, spmm_multi_long = 0;
   int sddmm_group = 0, sddmm_batches = 0, sddmm_blocked = -1, sddmm_block_cols = 0;
   int sddmm_fast = -1, sddmm_buffer_loads = -1, sddmm_rows = -1, sddmm_rows_blocks = 0;
@@ -74,27 +74,6 @@ struct SpmmShape {
 
 SpmmShape spmm_choose_shape(const SpmmArgs &a, int feat_tiles);
 
-// Per-wave block-major nonzero lists for the column-sweep kernel
-// (spmm_sweep.hip); device arrays, owned by the SpMM plan.
-struct SweepPlan {
-  int32_t generations = 0;    // launches needed to cover all rows
-  int32_t waves = 0;          // waves per launch, all resident at once
-  int32_t rows_per_wave = 0;  // R
-  int32_t *rows = nullptr;    // [generations * waves * R] row id or -1
-  int32_t *ptr = nullptr;     // [generations * waves + 1] list bounds
-  int32_t *col = nullptr;     // [nnz] column id of each list entry
-  int32_t *src = nullptr;     // [nnz] its position in the CSR arrays (for the value / weight)
-  uint8_t *lrow = nullptr;    // [nnz] which of the wave's R rows it belongs to
-  int64_t max_load = 0, mean_load = 0;  // nonzeros per wave
-};
-
-// indptr / order: host copies of the CSR row pointer and of the plan's row
-// list; seg: the plan's device bounds table with n_blocks >= 2 column blocks.
-// Leaves *sp empty (generations == 0) when the lists are not worth building.
-int sweep_build(const std::vector<int32_t> &indptr, const std::vector<int32_t> &order, const int32_t *seg,
-                int32_t n_blocks, const int32_t *indices, int64_t nnz, SweepPlan *sp);
-void sweep_free(SweepPlan *sp);
-int sweep_launch(const SweepPlan &sp, const SpmmArgs &a, int unroll, hipStream_t stream);
 int spmm_launch(const SpmmArgs &a, const SpmmShape &s, hipStream_t stream);
 
 // Several-rows-per-wave kernel with 16-byte gathers (spmm_multi.hip): single head, feature length a multiple

@@ -161,6 +161,10 @@ __device__ __forceinline__ void spmm_long_runs(const SpmmArgs &a, const FeatRows
             make_float4(v * x[r].x, v * x[r].y, v * x[r].z, v * x[r].w);
       }
     });
+    // The products were stored with one lane mapping and are read back with another.  LDS serves a wave's
+    // accesses in order; the fence and the barrier keep the compiler from moving the reads above the stores.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
     if (lane < TW) {
       static_for(std::make_integer_sequence<int, R>{}, [&](auto r) {
         constexpr int t = decltype(b)::value * R + decltype(r)::value;
@@ -169,6 +173,9 @@ __device__ __forceinline__ void spmm_long_runs(const SpmmArgs &a, const FeatRows
           if (NG * t + h < cnt) acc = acc + lds[decltype(r)::value * 256 + h * TW + lane];  // wave-uniform test
       });
     }
+    // ... and the next batch's stores below these reads
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
   };
 
   for (int it = wave; it < a.long_runs; it += n_waves) {

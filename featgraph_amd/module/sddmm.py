@@ -85,11 +85,14 @@ class SDDMMbase:
         compute_args = C.check_known_keys(compute_args, ("num_feat_partitions",), "compute_args")
         schedule_args = C.check_known_keys(
             schedule_args, ("num_feat_partitions", "num_cuda_blocks", "num_threads_per_cuda_block"), "schedule_args")
-        for args in (compute_args, schedule_args):
-            # feature tiling needs a cross-block reduction on a GPU; the reference's CUDA schedules
-            # refuse it too (op/vanilla_sddmm.py:79-80)
-            assert args.get("num_feat_partitions", 1) in (None, 0, 1), \
-                "the GPU schedule for sddmm does not support feat dimension tiling"
+        # num_feat_partitions (op/vanilla_sddmm.py:49, tests/test_module_sddmm.py:21-22): the x86 operator splits
+        # the reduction axis into P tiles; the reference's CUDA schedules refuse that (op/vanilla_sddmm.py:79-80)
+        # because their tiles would need a reduction across workgroups.  The kernels here tile long feature rows
+        # themselves (64 floats per tile, partial sums added tile by tile in one stream), so any P that divides the
+        # feature length is accepted; it does not change the tile width.
+        tiles = [int(args.get("num_feat_partitions") or 1) for args in (compute_args, schedule_args)]
+        if min(tiles) < 1:
+            raise ValueError("num_feat_partitions must be positive")
         if len(input_placeholders) != 2:
             raise ValueError("expected placeholders [SrcFeat, DstFeat]")
         for p in input_placeholders:
@@ -104,11 +107,16 @@ class SDDMMbase:
         H, D = self._heads_and_len(src_shape)
         if H * D < 1:
             raise ValueError("feature length must be positive")
+        for P in tiles:
+            if (H * D) % P != 0:
+                # the reference assumes this silently (op/vanilla_sddmm.py:49)
+                raise ValueError("feat_len %d is not a multiple of num_feat_partitions %d" % (H * D, P))
         return [src_shape, dst_shape], H, D
 
     def build(self, input_placeholders, compute_args, schedule_args):
         """Fix operand shapes and allocate the (zero-filled, reused) output: module/sddmm.py:72-92.
-        The reference's CUDA launch keys in schedule_args are accepted and ignored."""
+        The reference's CUDA launch keys in schedule_args are accepted and ignored; num_feat_partitions in either
+        dict must divide the feature length and is otherwise informational (see _parse_build)."""
         shapes, H, D = self._parse_build(input_placeholders, compute_args, schedule_args)
         self._input_shapes = shapes
         self._H, self._D = H, D

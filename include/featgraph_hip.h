@@ -16,7 +16,9 @@
  *     arrays (row list, bounds, run records; sizes are given with each plan).
  *   - Index arrays are int32, values and features float32, row-major, dense.
  *   - Kernels are enqueued on `stream` (a hipStream_t passed as void*, NULL =
- *     the default stream) and the call returns without synchronising.
+ *     the default stream) and the call returns without synchronising.  A plan
+ *     belongs to the device that was current when it was created; running it
+ *     with another device current returns FG_EINVAL.
  *   - Every output element is written by exactly one lane; results are
  *     deterministic and do not depend on launch shape or tile settings.
  *   - Return value: FG_OK or a negative FG_E* code; fg_last_error() then holds
@@ -188,7 +190,13 @@ FG_API int fg_sddmm_coo_mh_f32(int64_t nnz, const int32_t *row, const int32_t *c
 FG_API int fg_check_indices(int64_t n, const int32_t *idx, int64_t bound, int64_t *n_bad, void *stream);
 
 /*
- * Launch-shape overrides for tuning and tests.
+ * Launch-shape overrides for tuning and tests.  The store is process-global
+ * and unsynchronised: a single-threaded hook, not to be called while another
+ * thread is inside any entry point.  Some keys are read when a plan is created
+ * and some at every launch (noted per key); a plan created under one setting
+ * and launched under another stays correct, because every SpMM variant gives
+ * identical bits and every SDDMM variant results within float32 rounding; only
+ * the kernel choice changes.
  * Keys: "spmm.vec" (floats per lane: 1, 2, 4), "spmm.lpr" (lanes per row
  * slot: 8, 16, 32, 64), "spmm.unroll" (gathers in flight per lane: 4, 8, 16),
  * "spmm.scalar_path" (0/1: wave-per-row variant that keeps column ids in
@@ -199,9 +207,6 @@ FG_API int fg_check_indices(int64_t n, const int32_t *idx, int64_t bound, int64_
  * "spmm.pipeline" (0/1: wave-per-row kernel that keeps three rows in flight),
  * "spmm.pipe_blocks" (its grid size), "spmm.buffer_loads" (0/1: gather through
  * a buffer resource with scalar row offsets; needs a feature matrix below 4 GiB),
- * "spmm.sweep" (1: also build, and use, the per-wave block-major lists of the
- * experimental column-sweep kernel; read at plan creation and at launch),
- * "spmm.sweep_waves_per_cu" (its resident waves per CU),
  * "spmm.multi" (0/1: never / always use the several-rows-per-wave kernel where
  * it applies; by default it runs unless one of the shape keys above is set;
  * read at plan creation and at launch), "spmm.multi_blocks" (its grid size),

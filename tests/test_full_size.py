@@ -110,6 +110,107 @@ def test_c5_multihead_spmm_d64(c4):
     assert np.array_equal(out, want)
 
 
+# ---------------------------------------------------------------- every swept feature length at full size
+def _device_normal(shape, seed, dev):
+    """Seeded N(0,1) float32 operand drawn on the device (seconds faster than numpy at these sizes), plus its host copy."""
+    import torch
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    t = torch.randn(shape, dtype=torch.float32, device=dev, generator=g)
+    return t, t.cpu().numpy()
+
+
+@pytest.fixture(scope="module")
+def c2_spmm_module(c2):
+    return VanillaSpMMhip(c2)
+
+
+@pytest.fixture(scope="module")
+def c3_sddmm_module(c2):
+    coo = c2.tocoo()
+    return coo, VanillaSDDMMhip(coo)
+
+
+@pytest.mark.parametrize("F", [32, 128, 256, 512])
+def test_c2_spmm_bit_exact_at_every_swept_feature_length(c2, c2_spmm_module, F):
+    """Covers what only happens at full size: 15 column-block passes x F/64 tiles with carried sums, the
+    32768-column passes of the 32-float tile, more long runs than the workgroup clamp, 100 MB run tables."""
+    adj, module = c2, c2_spmm_module
+    n = adj.shape[0]
+    _say("SpMM c2 F=%d through VanillaSpMMhip: %s" % (F, module.lower_to_ir([placeholder((n, F))], {}, {})))
+    module.build([placeholder((n, F))], {}, {})
+    feat_dev, feat = _device_normal((n, F), 100 + F, module.ctx)
+    module.out_tvm.tensor.fill_(-1.0)
+    out = module.run([feat_dev]).asnumpy()
+    del feat_dev
+    want = ref.spmm_csr_x86(adj.indptr, adj.indices, adj.data, feat)
+    assert np.array_equal(out, want)
+
+
+@pytest.mark.parametrize("F", [32, 128, 256, 512])
+def test_c3_sddmm_at_every_swept_feature_length(c3_sddmm_module, F):
+    coo, module = c3_sddmm_module
+    n = coo.shape[0]
+    ph = [placeholder((n, F)), placeholder((n, F))]
+    _say("SDDMM c3 F=%d through VanillaSDDMMhip: %s" % (F, module.lower_to_ir(ph, {}, {})))
+    module.build(ph, {}, {})
+    src_dev, src = _device_normal((n, F), 200 + F, module.ctx)
+    dst_dev, dst = _device_normal((n, F), 300 + F, module.ctx)
+    module.out_tvm.tensor.fill_(-1.0)
+    out = module.run([src_dev, dst_dev]).asnumpy()
+    del src_dev, dst_dev
+    exact = ref.sddmm_f64(coo.row, coo.col, src, dst)
+    np.testing.assert_allclose(out, exact, rtol=RTOL, atol=ATOL)
+    # the strict serial float32 restatement (op/vanilla_sddmm.py:43-47) on the head and the tail of the list.  Its
+    # own rounding grows with the feature length (a 512-term sequential sum of magnitude ~20 is off by up to
+    # ~1e-4), so beyond 128 floats the bound is widened by exactly the restatement's distance from the exact value.
+    m = 2_000_000
+    for sl in (slice(0, m), slice(coo.nnz - m, coo.nnz)):
+        serial = ref.sddmm_x86(coo.row[sl], coo.col[sl], src, dst)
+        slack = np.abs(serial - exact[sl]) if F > 128 else 0.0
+        assert np.all(np.abs(out[sl] - serial) <= ATOL + RTOL * np.abs(serial) + slack)
+
+
+def test_c3_sddmm_on_a_shuffled_edge_list(c2):
+    """The same edges in a seeded random order: not row-sorted, so the plan re-orders the list by column block and
+    the edge-list kernels run; results must land at the caller's positions."""
+    import scipy.sparse
+    coo = c2.tocoo()
+    n, F = coo.shape[0], 64
+    perm = np.random.default_rng(17).permutation(coo.nnz)
+    shuffled = scipy.sparse.coo_matrix((coo.data[perm], (coo.row[perm], coo.col[perm])), shape=coo.shape)
+    module = VanillaSDDMMhip(shuffled)
+    ph = [placeholder((n, F)), placeholder((n, F))]
+    text = module.lower_to_ir(ph, {}, {})
+    _say("SDDMM c3 F=64, shuffled list: %s" % text)
+    assert "row runs" not in text
+    module.build(ph, {}, {})
+    src, dst = datasets.sddmm_operands(coo, F)
+    out = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
+    np.testing.assert_allclose(out, ref.sddmm_f64(shuffled.row, shuffled.col, src, dst), rtol=RTOL, atol=ATOL)
+    # against the sorted list's results, edge by edge: same dot products, possibly another summation tree
+    sorted_module = VanillaSDDMMhip(coo)
+    sorted_module.build(ph, {}, {})
+    base = sorted_module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
+    np.testing.assert_allclose(out, base[perm], rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("D", [32, 64])
+def test_c4_multihead_sddmm_longer_heads(c4, D):
+    """D = 64: 5 GB operands, beyond 32-bit buffer offsets, so the 64-bit addressing variant runs."""
+    coo = c4.tocoo()
+    n, H = coo.shape[0], 8
+    _say("multi-head SDDMM c4 H=8 D=%d through MultiHeadSDDMMhip" % D)
+    module = MultiHeadSDDMMhip(coo)
+    module.build([placeholder((n, H, D)), placeholder((n, H, D))], {}, {})
+    src_dev, src = _device_normal((n, H, D), 400 + D, module.ctx)
+    dst_dev, dst = _device_normal((n, H, D), 500 + D, module.ctx)
+    out = module.run([src_dev, dst_dev]).asnumpy()
+    del src_dev, dst_dev
+    assert out.shape == (coo.nnz, H)
+    np.testing.assert_allclose(out, ref.sddmm_mh(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
+
+
 def test_benchmark_commands_run_on_a_small_graph(tmp_path, capsys):
     import scipy.sparse
     from featgraph_amd.benchmark import bench_vanilla_sddmm, bench_vanilla_spmm

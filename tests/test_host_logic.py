@@ -128,3 +128,16 @@ def test_powerlaw_graph_shape_properties():
     has_self[rows[adj.indices == rows]] = True
     assert has_self.all()                                            # self-loops included
     assert adj.data.min() >= 0 and adj.data.max() < 1
+
+
+def test_reference_import_paths_resolve_to_this_implementation():
+    """`from featgraph.module import ...` / `from featgraph.util import ...` as the reference's callers write them
+    (tests/test_module_spmm.py:9, tests/test_module_sddmm.py:9, tests/test_util.py:5)."""
+    import featgraph
+    from featgraph.module import VanillaSDDMMcuda, VanillaSpMMcuda
+    from featgraph.module import VanillaSDDMMhip as S2, VanillaSpMMhip as S1
+    from featgraph.util import util_convert_csr_to_dds, util_partition_adj_coo_2d
+    assert VanillaSpMMcuda is S1 is VanillaSpMMhip and VanillaSDDMMcuda is S2 is VanillaSDDMMhip
+    assert util_convert_csr_to_dds is featgraph_amd.util.util_convert_csr_to_dds
+    assert util_partition_adj_coo_2d is featgraph_amd.util.util_partition_adj_coo_2d
+    assert featgraph.placeholder is placeholder and featgraph.nd is featgraph_amd.nd

@@ -288,22 +288,26 @@ def test_row_runs_on_awkward_structures(config_guard):
     np.testing.assert_allclose(_run_sddmm(one, src, dst), ref.sddmm_f64(one.row, one.col, src, dst), rtol=RTOL, atol=ATOL)
 
 
-# the reference's partitioned x86 test (tests/test_module_sddmm.py:16-41), partition arguments included
-@pytest.mark.parametrize("num_row_partitions,num_col_partitions", [(1, 1), (4, 4), (1, 7)])
-def test_partition_arguments_like_the_reference_x86_test(num_row_partitions, num_col_partitions):
+# the reference's partitioned x86 test (tests/test_module_sddmm.py:16-41) with its own parameter triples
+# (feat_len 128; num_feat_partitions, num_row_partitions, num_col_partitions) = (1,1,1), (4,1,1), (4,4,4), and two more
+@pytest.mark.parametrize("num_feat_partitions,num_row_partitions,num_col_partitions",
+                         [(1, 1, 1), (4, 1, 1), (4, 4, 4), (1, 4, 4), (8, 1, 7)])
+def test_partition_arguments_like_the_reference_x86_test(num_feat_partitions, num_row_partitions, num_col_partitions):
     coo = reference_test_matrix("coo", seed=0)
     rng = np.random.default_rng(1)
     src = rng.random((coo.shape[1], 128)).astype("float32")
     dst = rng.random((coo.shape[0], 128)).astype("float32")
     module = VanillaSDDMMhip(coo, num_row_partitions, num_col_partitions)
-    module.build([placeholder(src.shape), placeholder(dst.shape)], {}, {})
-    text = module.lower_to_ir([placeholder(src.shape), placeholder(dst.shape)], {}, {})
+    compute_args = {"num_feat_partitions": num_feat_partitions}
+    schedule_args = {"num_feat_partitions": num_feat_partitions}
+    module.build([placeholder(src.shape), placeholder(dst.shape)], compute_args, schedule_args)
+    text = module.lower_to_ir([placeholder(src.shape), placeholder(dst.shape)], compute_args, schedule_args)
     assert ("%d column blocks" % num_col_partitions in text) == (num_col_partitions > 1)
     out = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
     if num_row_partitions != 1 or num_col_partitions != 1:
         out = out[module.edge_mapping]
     np.testing.assert_allclose((src[coo.col] * dst[coo.row]).sum(axis=-1), out, rtol=1e-4, atol=1e-4)
-    np.testing.assert_allclose(out, ref.sddmm_x86(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(out, ref.sddmm_x86(coo.row, coo.col, src, dst, num_feat_partitions), rtol=RTOL, atol=ATOL)
 
 
 def test_module_surface(adj_127x255):
@@ -312,8 +316,8 @@ def test_module_surface(adj_127x255):
     assert module.target == "hip"
     with pytest.raises(AssertionError):
         module.edge_mapping                                           # module/sddmm.py:155-156: no partitioning asked for
-    with pytest.raises(AssertionError):
-        module.build([placeholder((coo.shape[1], 8)), placeholder((coo.shape[0], 8))], {"num_feat_partitions": 2}, {})
+    with pytest.raises(ValueError):                                   # 8 floats do not split into 3 tiles
+        module.build([placeholder((coo.shape[1], 8)), placeholder((coo.shape[0], 8))], {"num_feat_partitions": 3}, {})
     with pytest.raises(AssertionError):
         module.build([placeholder((coo.shape[1], 8)), placeholder((coo.shape[0], 16))], {}, {})
     module.build([placeholder((coo.shape[1], 8)), placeholder((coo.shape[0], 8))], {}, {})
