@@ -1,0 +1,102 @@
+// Measurement aid: how fast the part serves the gather pattern of the SpMM / SDDMM kernels when nothing else
+// is asked of it.
+//
+// fg_probe_gather_f32 issues n_gathers row gathers per feature tile with the kernels' own shape: a group of
+// tile/4 lanes fetches one row's tile with 16-byte loads (a 64-float tile: four rows per wave instruction),
+// sixteen gathers in flight per lane, the rows of one launch drawn from one band of `band_rows` consecutive
+// rows, one launch per band and tile, bands in ascending order.  What it leaves out is everything a real
+// operator adds: no index or value stream (row numbers come from a per-group random-number recurrence), no
+// sums carried between launches, no ordered accumulation, no output.  The time it takes is therefore a floor
+// for any kernel that moves the same rows through the same cache hierarchy with the same blocking, and
+// bench.py reports operator time against it.
+#include <algorithm>
+
+#include "common.hpp"
+
+namespace {
+
+constexpr int kProbeBlocks = 4096;  // workgroups per launch
+
+template <int G>
+__global__ __launch_bounds__(fg::kBlockThreads) void probe_gather_kernel(const float *feat, uint32_t row_bytes,
+                                                                         uint32_t tile_byte0, uint32_t band_lo,
+                                                                         uint32_t band_rows, int iters,
+                                                                         uint32_t bytes, float *sink) {
+  constexpr int U = 16;
+  const int lane = threadIdx.x & (fg::kWaveSize - 1);
+  const int gl = lane & (G - 1), g = lane / G;
+  const uint32_t wave = blockIdx.x * fg::kWavesPerBlock + (threadIdx.x >> 6);
+  uint32_t s = wave * 2654435761u + static_cast<uint32_t>(g) * 40503u + band_lo * 97u + 12345u;
+  float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(feat), 0, static_cast<int>(bytes), 0x00020000);
+  for (int it = 0; it < iters; ++it) {
+    float4 x[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      s = s * 1664525u + 1013904223u;
+      const uint32_t r = band_lo + (s >> 8) % band_rows;
+      const uint32_t off = r * row_bytes + tile_byte0 + static_cast<uint32_t>(gl) * 16u;
+      x[u] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, static_cast<int>(off), 0, 0));
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      acc.x += x[u].x;
+      acc.y += x[u].y;
+      acc.z += x[u].z;
+      acc.w += x[u].w;
+    }
+  }
+  // keeps the loads alive; finite feature values never produce this sum
+  if (acc.x + acc.y + acc.z + acc.w == __builtin_inff()) sink[0] = acc.x;
+}
+
+}  // namespace
+
+extern "C" int fg_probe_gather_f32(const float *feat, int64_t n_rows, int32_t F, int32_t tile, int32_t band_rows,
+                                   int64_t n_gathers, float *sink, void *stream) {
+  if (!feat || !sink) return fg::fail(FG_EINVAL, "feat or sink is null");
+  if (n_rows < 1 || F < 4 || F % 4 != 0) return fg::fail(FG_EINVAL, "need n_rows >= 1 and F a positive multiple of 4");
+  if (tile != 16 && tile != 32 && tile != 64) return fg::fail(FG_EINVAL, "tile = %d is not one of 16, 32, 64", tile);
+  if (F % tile != 0) return fg::fail(FG_EINVAL, "F = %d is not a multiple of the tile width %d", F, tile);
+  if (band_rows < 1 || n_gathers < 0) return fg::fail(FG_EINVAL, "band_rows must be positive, n_gathers non-negative");
+  if (n_rows * F * 4 >= (int64_t{1} << 32))
+    return fg::fail(FG_EUNSUPPORTED, "the probe addresses the matrix with 32-bit offsets: below 4 GiB only");
+  if (!fg::aligned_to(feat, 16)) return fg::fail(FG_EINVAL, "feat must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int G = tile / 4;
+  const int64_t passes = (n_rows + band_rows - 1) / band_rows;
+  const int blocks = kProbeBlocks;
+  const int64_t per_iter = static_cast<int64_t>(blocks) * fg::kWavesPerBlock * (fg::kWaveSize / G) * 16;
+  const int iters = static_cast<int>(std::max<int64_t>(1, (n_gathers / passes + per_iter / 2) / per_iter));
+  const uint32_t bytes = static_cast<uint32_t>(n_rows * F * 4);
+  for (int t = 0; t < F / tile; ++t) {
+    for (int64_t p = 0; p < passes; ++p) {
+      const uint32_t lo = static_cast<uint32_t>(p * band_rows);
+      const uint32_t rows = static_cast<uint32_t>(std::min<int64_t>(band_rows, n_rows - p * band_rows));
+      const uint32_t byte0 = static_cast<uint32_t>(t) * tile * 4u;
+      if (G == 4)
+        probe_gather_kernel<4><<<dim3(blocks), dim3(fg::kBlockThreads), 0, st>>>(feat, F * 4u, byte0, lo, rows, iters,
+                                                                                bytes, sink);
+      else if (G == 8)
+        probe_gather_kernel<8><<<dim3(blocks), dim3(fg::kBlockThreads), 0, st>>>(feat, F * 4u, byte0, lo, rows, iters,
+                                                                                bytes, sink);
+      else
+        probe_gather_kernel<16><<<dim3(blocks), dim3(fg::kBlockThreads), 0, st>>>(feat, F * 4u, byte0, lo, rows,
+                                                                                 iters, bytes, sink);
+    }
+  }
+  FG_HIP_TRY(hipGetLastError());
+  return FG_OK;
+}
+
+// Gathers that one call of fg_probe_gather_f32 with these arguments issues per feature tile (the request is
+// rounded to whole iterations of the launch grid).
+extern "C" int64_t fg_probe_gather_count(int64_t n_rows, int32_t tile, int32_t band_rows, int64_t n_gathers) {
+  if (n_rows < 1 || band_rows < 1 || (tile != 16 && tile != 32 && tile != 64) || n_gathers < 0) return -1;
+  const int G = tile / 4;
+  const int64_t passes = (n_rows + band_rows - 1) / band_rows;
+  const int64_t per_iter = int64_t{kProbeBlocks} * fg::kWavesPerBlock * (fg::kWaveSize / G) * 16;
+  const int64_t iters = std::max<int64_t>(1, (n_gathers / passes + per_iter / 2) / per_iter);
+  return passes * iters * per_iter;
+}

@@ -190,6 +190,24 @@ FG_API int fg_sddmm_coo_mh_f32(int64_t nnz, const int32_t *row, const int32_t *c
 FG_API int fg_check_indices(int64_t n, const int32_t *idx, int64_t bound, int64_t *n_bad, void *stream);
 
 /*
+ * Measurement aid (no counterpart in the reference): the gather pattern of the
+ * SpMM / SDDMM kernels with everything else left out.  Per feature tile of
+ * `tile` floats (16, 32 or 64; F a multiple of it) it gathers about n_gathers
+ * random rows of feat [n_rows, F] with 16-byte loads, tile/4 lanes per row,
+ * sixteen gathers in flight per lane, one launch per band of band_rows
+ * consecutive rows and per tile, bands in ascending order; no index or value
+ * stream, no sums, no output (sink, one float, is never written for finite
+ * features).  Its time is a floor for any kernel that moves the same rows
+ * through the caches with the same blocking.  fg_probe_gather_count returns
+ * the gathers per tile that such a call really issues (the request is rounded
+ * to whole iterations of the grid), or -1 for arguments the probe rejects.
+ * The matrix must span less than 4 GiB.
+ */
+FG_API int fg_probe_gather_f32(const float *feat, int64_t n_rows, int32_t F, int32_t tile, int32_t band_rows,
+                               int64_t n_gathers, float *sink, void *stream);
+FG_API int64_t fg_probe_gather_count(int64_t n_rows, int32_t tile, int32_t band_rows, int64_t n_gathers);
+
+/*
  * Launch-shape overrides for tuning and tests.  The store is process-global
  * and unsynchronised: a single-threaded hook, not to be called while another
  * thread is inside any entry point.  Some keys are read when a plan is created
