@@ -21,6 +21,8 @@ SIGNATURES = {
     "fg_spmm_plan_row_order": (ctypes.c_int, [_p, _p, ctypes.POINTER(_i32)]),
     "fg_spmm_csr_f32": (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _p]),
     "fg_spmm_csr_noalloc_f32": (ctypes.c_int, [_i64, _i64, _i64, _p, _p, _p, _p, _p, _i32, _p]),
+    "fg_spmm_csr_general_f32": (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _i32, _p]),
+    "fg_sddmm_coo_general_f32": (ctypes.c_int, [_i64, _p, _p, _p, _p, _p, _i32, _i32, _p]),
     "fg_spmm_csr_mh_f32": (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _i32, _p]),
     "fg_sddmm_coo_f32": (ctypes.c_int, [_i64, _p, _p, _p, _p, _p, _i32, _p]),
     "fg_sddmm_coo_mh_f32": (ctypes.c_int, [_i64, _p, _p, _p, _p, _p, _i32, _i32, _p]),

@@ -565,6 +565,35 @@ int fg_spmm_csr_mh_f32(const fg_spmm_plan *plan, const float *feat, const float 
   return FG_OK;
 }
 
+int fg_spmm_csr_general_f32(const fg_spmm_plan *plan, const float *feat, const float *vals, float *out, int32_t F,
+                            int32_t msg, int32_t reduce, void *stream) {
+  if (!plan) return fg::fail(FG_EINVAL, "plan is null");
+  if (int rc = check_heads(1, F)) return rc;
+  if (int rc = check_device(plan->device)) return rc;
+  if (msg < FG_MSG_MUL || msg > FG_MSG_COPY_U) return fg::fail(FG_EINVAL, "msg = %d is not an FG_MSG_* code", msg);
+  if (reduce < FG_REDUCE_SUM || reduce > FG_REDUCE_MEAN)
+    return fg::fail(FG_EINVAL, "reduce = %d is not an FG_REDUCE_* code", reduce);
+  if (plan->n_rows > 0 && !out) return fg::fail(FG_EINVAL, "out is null");
+  if (plan->nnz > 0 && (!feat || (!vals && msg != FG_MSG_COPY_U)))
+    return fg::fail(FG_EINVAL, "feat or edge values are null");
+  if (plan->n_rows == 0) return FG_OK;
+  const int32_t *lo = plan->seg;  // whole rows, in the plan's visiting order
+  const int32_t *hi = plan->seg + static_cast<int64_t>(plan->n_blocks) * plan->n_rows;
+  return fg::spmm_general_launch(plan->row_order, lo, hi, plan->indices, vals, feat, out,
+                                 static_cast<int32_t>(plan->n_rows), F, msg, reduce, static_cast<hipStream_t>(stream));
+}
+
+int fg_sddmm_coo_general_f32(int64_t nnz, const int32_t *row, const int32_t *col, const float *src, const float *dst,
+                             float *out, int32_t F, int32_t edge_op, void *stream) {
+  if (edge_op == FG_EDGE_DOT) return fg_sddmm_coo_f32(nnz, row, col, src, dst, out, F, stream);
+  if (edge_op < FG_EDGE_DOT || edge_op > FG_EDGE_DIV)
+    return fg::fail(FG_EINVAL, "edge_op = %d is not an FG_EDGE_* code", edge_op);
+  if (nnz < 0) return fg::fail(FG_EINVAL, "nnz = %lld is negative", (long long)nnz);
+  if (int rc = check_heads(1, F)) return rc;
+  if (nnz > 0 && (!row || !col || !src || !dst || !out)) return fg::fail(FG_EINVAL, "a data pointer is null");
+  return fg::sddmm_elementwise_launch(row, col, src, dst, out, nnz, F, edge_op, static_cast<hipStream_t>(stream));
+}
+
 int fg_sddmm_coo_f32(int64_t nnz, const int32_t *row, const int32_t *col, const float *src, const float *dst,
                      float *out, int32_t F, void *stream) {
   return fg_sddmm_coo_mh_f32(nnz, row, col, src, dst, out, 1, F, stream);

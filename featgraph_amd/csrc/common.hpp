@@ -145,6 +145,13 @@ int sddmm_rows_launch(const int32_t *seg, const int32_t *row_order, int32_t n_ro
                       const int32_t *col, const float *src, const float *dst, float *out, int64_t src_bytes,
                       int64_t dst_bytes, int32_t F, hipStream_t stream);
 
+// Generalised operators (general.hip): msg / reduce / op are the FG_MSG_* / FG_REDUCE_* / FG_EDGE_* codes.
+int spmm_general_launch(const int32_t *row_order, const int32_t *seg_lo, const int32_t *seg_hi, const int32_t *indices,
+                        const float *vals, const float *feat, float *out, int32_t n_rows, int32_t F, int msg,
+                        int reduce, hipStream_t stream);
+int sddmm_elementwise_launch(const int32_t *row, const int32_t *col, const float *src, const float *dst, float *out,
+                             int64_t nnz, int32_t F, int op, hipStream_t stream);
+
 inline bool aligned_to(const void *p, uintptr_t bytes) { return (reinterpret_cast<uintptr_t>(p) & (bytes - 1)) == 0; }
 
 inline int pow2_ceil(int x) {

@@ -1,2 +1,3 @@
 from .sddmm import VanillaSDDMMhip, MultiHeadSDDMMhip
 from .spmm import VanillaSpMMhip, MultiHeadSpMMhip
+from .general import GeneralizedSpMMhip, GeneralizedSDDMMhip, VanillaSpMMGradhip

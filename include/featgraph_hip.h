@@ -120,6 +120,32 @@ FG_API int fg_spmm_csr_noalloc_f32(int64_t n_rows, int64_t n_cols, int64_t nnz, 
                                    int32_t F, void *stream);
 
 /*
+ * Generalised SpMM: the message and reduce slots of the reference's operator
+ * template (op/vanilla_spmm.py:46-53: msgfunc forms adj_val * feat_val and
+ * folds it with te.sum) opened to the other operators of "generalized SpMM"
+ * (README.md:6).  The reference itself ships only (FG_MSG_MUL, FG_REDUCE_SUM).
+ *   term(e, f) = msg(feat[indices[e], f], vals[e])
+ *   Out[r, f]  = fold of the row's terms in CSR order
+ * FG_REDUCE_SUM starts from +0; MAX / MIN fold as acc = (t > acc) ? t : acc;
+ * MEAN is the sum divided by the row's degree (one rounded division).  Rows
+ * without nonzeros give 0 under every reducer.  One rounded operation per
+ * message and per fold step, so (MUL, SUM) equals fg_spmm_csr_f32 bit for bit.
+ * vals may be null for FG_MSG_COPY_U.  Single launch over whole rows in the
+ * plan's row order.
+ */
+#define FG_MSG_MUL 0
+#define FG_MSG_ADD 1
+#define FG_MSG_SUB 2
+#define FG_MSG_DIV 3
+#define FG_MSG_COPY_U 4
+#define FG_REDUCE_SUM 0
+#define FG_REDUCE_MAX 1
+#define FG_REDUCE_MIN 2
+#define FG_REDUCE_MEAN 3
+FG_API int fg_spmm_csr_general_f32(const fg_spmm_plan *plan, const float *feat, const float *vals, float *out,
+                                   int32_t F, int32_t msg, int32_t reduce, void *stream);
+
+/*
  * Multi-head generalised SpMM (no counterpart in the reference, whose
  * op/__init__.py:1-5 exports vanilla operators only; same message function as
  * op/vanilla_spmm.py:46-53 with a per-head weight):
@@ -138,6 +164,20 @@ FG_API int fg_spmm_csr_mh_f32(const fg_spmm_plan *plan, const float *feat, const
  */
 FG_API int fg_sddmm_coo_f32(int64_t nnz, const int32_t *row, const int32_t *col, const float *src, const float *dst,
                      float *out, int32_t F, void *stream);
+
+/*
+ * Generalised SDDMM: the edge-function slot of op/vanilla_sddmm.py:43-47.
+ * FG_EDGE_DOT is fg_sddmm_coo_f32 (out [nnz]); the other operators keep the
+ * feature axis: Out[e, f] = src[col[e], f] op dst[row[e], f], out [nnz, F],
+ * one rounded operation per element.
+ */
+#define FG_EDGE_DOT 0
+#define FG_EDGE_ADD 1
+#define FG_EDGE_SUB 2
+#define FG_EDGE_MUL 3
+#define FG_EDGE_DIV 4
+FG_API int fg_sddmm_coo_general_f32(int64_t nnz, const int32_t *row, const int32_t *col, const float *src,
+                                    const float *dst, float *out, int32_t F, int32_t edge_op, void *stream);
 
 /*
  * Cache-blocking schedule for one COO edge list; takes the place that

@@ -269,3 +269,93 @@ int fgref_spmm_mh(int64_t n_dst, int64_t H, int64_t D, const int32_t *indptr, co
   }
   return FGREF_OK;
 }
+
+/* Generalised SpMM: the message and reduce slots of the reference's SpMM template
+ * (op/vanilla_spmm.py:46-53: msgfunc builds adj_val * feat_val and folds it with
+ * te.sum) opened to the operators that README.md:6 calls "generalized SpMM".
+ * The reference ships only the (mul, sum) instance; the others are defined here:
+ *   term(e, f) = msg(Src[indices[e], f], vals[e])   msg: 0 u*e, 1 u+e, 2 u-e, 3 u/e, 4 u
+ *   Out[r, f]  = fold over e in CSR order           reduce: 0 sum (from +0), 1 max, 2 min,
+ *                                                   3 mean = sum / degree (one rounded division)
+ * max / min fold as acc = (t > acc) ? t : acc from the row's first term, so the
+ * result (including the sign of a zero) is fixed by the order.  Rows without
+ * nonzeros give 0 under every reducer.  (mul, sum) is fgref_spmm_csr_x86 bit for bit. */
+static inline float fgref_msg(int msg, float u, float e) {
+  switch (msg) {
+    case 0: return u * e;
+    case 1: return u + e;
+    case 2: return u - e;
+    case 3: return u / e;
+    default: return u;
+  }
+}
+
+int fgref_spmm_general(int64_t n_dst, int64_t F, const int32_t *indptr, const int32_t *indices, const float *vals,
+                       const float *src, float *out, int msg, int reduce) {
+  if (n_dst < 0 || F <= 0 || msg < 0 || msg > 4 || reduce < 0 || reduce > 3) return FGREF_EINVAL;
+#pragma omp parallel for schedule(dynamic, 64)
+  for (int64_t r = 0; r < n_dst; ++r) {
+    float *acc = out + r * F;
+    const int64_t lo = indptr[r], hi = indptr[r + 1];
+    for (int64_t f = 0; f < F; ++f) acc[f] = 0.0f;
+    for (int64_t e = lo; e < hi; ++e) {
+      const float *x = src + (int64_t)indices[e] * F;
+      const float v = msg == 4 ? 0.0f : vals[e];
+      for (int64_t f = 0; f < F; ++f) {
+        const float t = fgref_msg(msg, x[f], v);
+        if (reduce == 0 || reduce == 3)
+          acc[f] = acc[f] + t;
+        else if (e == lo)
+          acc[f] = t;
+        else if (reduce == 1)
+          acc[f] = (t > acc[f]) ? t : acc[f];
+        else
+          acc[f] = (t < acc[f]) ? t : acc[f];
+      }
+    }
+    if (reduce == 3 && hi > lo) {
+      const float n = (float)(hi - lo);
+      for (int64_t f = 0; f < F; ++f) acc[f] = acc[f] / n;
+    }
+  }
+  return FGREF_OK;
+}
+
+/* Generalised SDDMM with an elementwise edge function (the edgefunc slot of
+ * op/vanilla_sddmm.py:43-47 without its reduction over k):
+ * Out[e, f] = Src[col[e], f] op Dst[row[e], f], op: 1 add, 2 sub, 3 mul, 4 div.
+ * (op 0, the dot product, is fgref_sddmm_x86.) */
+int fgref_sddmm_general(int64_t nnz, int64_t F, const int32_t *row, const int32_t *col, const float *src,
+                        const float *dst, float *out, int op) {
+  if (nnz < 0 || F <= 0 || op < 1 || op > 4) return FGREF_EINVAL;
+#pragma omp parallel for schedule(static)
+  for (int64_t e = 0; e < nnz; ++e) {
+    const float *a = src + (int64_t)col[e] * F, *b = dst + (int64_t)row[e] * F;
+    float *o = out + e * F;
+    for (int64_t f = 0; f < F; ++f)
+      o[f] = op == 1 ? a[f] + b[f] : op == 2 ? a[f] - b[f] : op == 3 ? a[f] * b[f] : a[f] / b[f];
+  }
+  return FGREF_OK;
+}
+
+/* Edge softmax (not in the reference; it is the step between the attention
+ * scores of multi-head SDDMM and the weights of multi-head SpMM in a GAT layer):
+ * for every destination row r and head h, over the row's edges in CSR order,
+ * Out[e, h] = exp(S[e, h] - max_r,h) / sum_e' exp(S[e', h] - max_r,h).
+ * Computed in binary64 and rounded once, so it serves as the exact value that a
+ * float32 kernel is held to within tolerance. */
+#include <math.h>
+int fgref_edge_softmax(int64_t n_dst, int64_t H, const int32_t *indptr, const float *scores, float *out) {
+  if (n_dst < 0 || H <= 0) return FGREF_EINVAL;
+#pragma omp parallel for schedule(dynamic, 64)
+  for (int64_t r = 0; r < n_dst; ++r) {
+    const int64_t lo = indptr[r], hi = indptr[r + 1];
+    for (int64_t h = 0; h < H; ++h) {
+      double m = -INFINITY, sum = 0.0;
+      for (int64_t e = lo; e < hi; ++e) m = scores[e * H + h] > m ? scores[e * H + h] : m;
+      for (int64_t e = lo; e < hi; ++e) sum += exp((double)scores[e * H + h] - m);
+      for (int64_t e = lo; e < hi; ++e) out[e * H + h] = (float)(exp((double)scores[e * H + h] - m) / sum);
+    }
+  }
+  return FGREF_OK;
+}

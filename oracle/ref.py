@@ -32,7 +32,8 @@ def lib():
             build()
         _lib = ctypes.CDLL(_LIB_PATH)
         for name in ("fgref_spmm_csr_x86", "fgref_spmm_dds_x86", "fgref_sddmm_x86", "fgref_sddmm_x86_fast",
-                     "fgref_spmm_csr_f64", "fgref_sddmm_f64", "fgref_sddmm_mh", "fgref_spmm_mh"):
+                     "fgref_spmm_csr_f64", "fgref_sddmm_f64", "fgref_sddmm_mh", "fgref_spmm_mh", "fgref_spmm_general",
+                     "fgref_sddmm_general", "fgref_edge_softmax"):
             getattr(_lib, name).restype = ctypes.c_int
     return _lib
 
@@ -150,4 +151,44 @@ def spmm_mh(indptr, indices, w, src):
     out = np.empty((n_dst, H, D), dtype=np.float32)
     _check(lib().fgref_spmm_mh(_i64(n_dst), _i64(H), _i64(D), _ptr(indptr), _ptr(indices), _ptr(w), _ptr(src),
                                _ptr(out)), "fgref_spmm_mh")
+    return out
+
+
+MSG_OPS = {"mul": 0, "add": 1, "sub": 2, "div": 3, "copy_u": 4}
+REDUCE_OPS = {"sum": 0, "max": 1, "min": 2, "mean": 3}
+EDGE_OPS = {"dot": 0, "add": 1, "sub": 2, "mul": 3, "div": 4}
+
+
+def spmm_general(indptr, indices, vals, src, msg="mul", reduce="sum"):
+    """Generalised SpMM: fold of msg(src[col], val) over each row in CSR order (see fgref_spmm_general)."""
+    indptr, indices, vals = _arr(indptr, np.int32), _arr(indices, np.int32), _arr(vals, np.float32)
+    src = _arr(src, np.float32)
+    n_dst, F = indptr.shape[0] - 1, src.shape[1]
+    out = np.empty((n_dst, F), dtype=np.float32)
+    _check(lib().fgref_spmm_general(_i64(n_dst), _i64(F), _ptr(indptr), _ptr(indices), _ptr(vals), _ptr(src),
+                                    _ptr(out), ctypes.c_int(MSG_OPS[msg]), ctypes.c_int(REDUCE_OPS[reduce])),
+           "fgref_spmm_general")
+    return out
+
+
+def sddmm_general(row, col, src, dst, op):
+    """Elementwise edge function: out[e, :] = src[col[e], :] op dst[row[e], :]; 'dot' is sddmm_x86."""
+    if op == "dot":
+        return sddmm_x86(row, col, src, dst)
+    row, col = _arr(row, np.int32), _arr(col, np.int32)
+    src, dst = _arr(src, np.float32), _arr(dst, np.float32)
+    nnz, F = row.shape[0], src.shape[1]
+    out = np.empty((nnz, F), dtype=np.float32)
+    _check(lib().fgref_sddmm_general(_i64(nnz), _i64(F), _ptr(row), _ptr(col), _ptr(src), _ptr(dst), _ptr(out),
+                                     ctypes.c_int(EDGE_OPS[op])), "fgref_sddmm_general")
+    return out
+
+
+def edge_softmax(indptr, scores):
+    """Softmax of scores [nnz, H] over each destination row's edges, per head (binary64 inside)."""
+    indptr, scores = _arr(indptr, np.int32), _arr(scores, np.float32)
+    n_dst, H = indptr.shape[0] - 1, scores.shape[1]
+    out = np.empty_like(scores)
+    _check(lib().fgref_edge_softmax(_i64(n_dst), _i64(H), _ptr(indptr), _ptr(scores), _ptr(out)),
+           "fgref_edge_softmax")
     return out

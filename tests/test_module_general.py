@@ -1,0 +1,146 @@
+"""GPU parity of the generalised operators (message / reduce / edge-function slots) and of the SpMM backward,
+through the module layer and the C ABI, against the CPU checker (oracle/) and numpy closed forms.
+
+Bars: generalised SpMM bit-exact (the kernel folds each row in CSR order with one rounded operation per step, as
+the checker does); elementwise SDDMM bit-exact (one rounded operation per element); the backward inherits the
+bars of the two vanilla kernels it is made of.
+"""
+import numpy as np
+import pytest
+import scipy.sparse
+
+from conftest import reference_test_matrix
+from featgraph_amd import datasets, nd, placeholder
+from featgraph_amd.module import (GeneralizedSDDMMhip, GeneralizedSpMMhip, VanillaSDDMMhip, VanillaSpMMGradhip,
+                                  VanillaSpMMhip)
+from oracle import ref
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-5, 1e-4
+MSGS = ["mul", "add", "sub", "div", "copy_u"]
+REDUCES = ["sum", "max", "min", "mean"]
+
+
+def _run_general_spmm(adj, feat, msg, reduce):
+    module = GeneralizedSpMMhip(adj, msg, reduce)
+    module.build([placeholder(feat.shape)], {}, {})
+    module.out_tvm.tensor.fill_(7.0)                      # every element must be overwritten, empty rows too
+    return module.run([nd.array(feat, module.ctx)]).asnumpy()
+
+
+@pytest.mark.parametrize("msg", MSGS)
+@pytest.mark.parametrize("reduce", REDUCES)
+def test_every_message_and_reducer_on_the_reference_matrix_family(adj_127x255, msg, reduce):
+    adj = adj_127x255.copy()
+    adj.data = adj.data + np.float32(0.25)                # keep divisors away from zero
+    for F in (128, 5):                                    # float4 lanes; scalar lanes with a partial tile
+        feat = np.random.default_rng(F).standard_normal((adj.shape[1], F), dtype=np.float32)
+        out = _run_general_spmm(adj, feat, msg, reduce)
+        assert np.array_equal(out, ref.spmm_general(adj.indptr, adj.indices, adj.data, feat, msg, reduce)), F
+
+
+@pytest.mark.parametrize("reduce", REDUCES)
+def test_hub_rows_empty_rows_and_unsorted_duplicate_columns(reduce):
+    adj = datasets.config_graph("c2-mini")                # rows of up to 3,000 nonzeros
+    feat = datasets.spmm_operands(adj, 64)
+    for msg in ("mul", "add"):
+        out = _run_general_spmm(adj, feat, msg, reduce)
+        assert np.array_equal(out, ref.spmm_general(adj.indptr, adj.indices, adj.data, feat, msg, reduce)), msg
+    # rows 1 and 3 empty, row 2 with descending and repeated columns: the fold follows the stored order
+    raw = scipy.sparse.csr_matrix((np.array([2, 1, 4, 3, 5], np.float32), np.array([3, 1, 1, 0, 2], np.int32),
+                                   np.array([0, 1, 1, 4, 4, 5], np.int32)), shape=(5, 4))
+    small = np.random.default_rng(9).standard_normal((4, 12), dtype=np.float32)
+    out = _run_general_spmm(raw, small, "sub", reduce)
+    assert np.array_equal(out, ref.spmm_general(raw.indptr, raw.indices, raw.data, small, "sub", reduce))
+    assert np.all(out[[1, 3]] == 0)
+
+
+def test_mul_sum_is_the_vanilla_kernel_and_max_min_match_numpy(adj_127x255):
+    adj = adj_127x255
+    feat = np.random.default_rng(2).standard_normal((adj.shape[1], 96), dtype=np.float32)
+    vanilla = VanillaSpMMhip(adj)
+    vanilla.build([placeholder(feat.shape)], {}, {})
+    assert np.array_equal(_run_general_spmm(adj, feat, "mul", "sum"), vanilla.run([nd.array(feat, vanilla.ctx)]).asnumpy())
+    rows = np.flatnonzero(np.diff(adj.indptr) > 0)
+    terms = feat[adj.indices]                              # copy_u: the terms are the gathered rows themselves
+    assert np.array_equal(_run_general_spmm(adj, feat, "copy_u", "max")[rows],
+                          np.maximum.reduceat(terms, adj.indptr[rows], axis=0))
+    assert np.array_equal(_run_general_spmm(adj, feat, "copy_u", "min")[rows],
+                          np.minimum.reduceat(terms, adj.indptr[rows], axis=0))
+
+
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
+def test_elementwise_edge_functions(op):
+    coo = reference_test_matrix("coo", seed=4)
+    rng = np.random.default_rng(5)
+    for F in (128, 6, 1):
+        src = rng.standard_normal((coo.shape[1], F), dtype=np.float32)
+        dst = rng.standard_normal((coo.shape[0], F), dtype=np.float32) + np.float32(3.0)
+        module = GeneralizedSDDMMhip(coo, op)
+        module.build([placeholder(src.shape), placeholder(dst.shape)], {}, {})
+        out = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
+        assert out.shape == (coo.nnz, F)
+        assert np.array_equal(out, ref.sddmm_general(coo.row, coo.col, src, dst, op)), F
+        a, b = src[coo.col], dst[coo.row]
+        assert np.array_equal(out, {"add": a + b, "sub": a - b, "mul": a * b, "div": a / b}[op])
+
+
+def test_dot_edge_function_is_the_vanilla_module():
+    coo = reference_test_matrix("coo", seed=4)
+    src, dst = datasets.sddmm_operands(coo, 128)
+    outs = []
+    for module in (GeneralizedSDDMMhip(coo, "dot"), VanillaSDDMMhip(coo)):
+        module.build([placeholder(src.shape), placeholder(dst.shape)], {}, {})
+        outs.append(module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy())
+    assert outs[0].shape == (coo.nnz,) and np.array_equal(outs[0], outs[1])
+
+
+def test_elementwise_edge_function_on_a_large_edge_list():
+    adj = datasets.config_graph("c4-mini")
+    coo = adj.tocoo()
+    src, dst = datasets.sddmm_operands(coo, 32)
+    module = GeneralizedSDDMMhip(coo, "mul")
+    module.build([placeholder(src.shape), placeholder(dst.shape)], {}, {})
+    out = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
+    assert np.array_equal(out, src[coo.col] * dst[coo.row])
+    # summing the elementwise products over the feature axis is the dot product, up to summation order
+    np.testing.assert_allclose(out.astype(np.float64).sum(-1), ref.sddmm_f64(coo.row, coo.col, src, dst),
+                               rtol=RTOL, atol=ATOL)
+
+
+def test_bad_operator_names_and_codes():
+    from featgraph_amd import _lib
+    adj = reference_test_matrix("csr", seed=0)
+    with pytest.raises(ValueError):
+        GeneralizedSpMMhip(adj, "pow", "sum")
+    with pytest.raises(ValueError):
+        GeneralizedSpMMhip(adj, "mul", "prod")
+    with pytest.raises(ValueError):
+        GeneralizedSDDMMhip(adj.tocoo(), "xor")
+    L = _lib.lib()
+    assert L.fg_sddmm_coo_general_f32(4, 8, 8, 8, 8, 8, 4, 9, None) == -1
+    assert L.fg_spmm_csr_general_f32(None, None, None, None, 4, 0, 0, None) == -1
+
+
+# ---------------------------------------------------------------- backward of vanilla SpMM
+@pytest.mark.parametrize("name,F", [("c2-mini", 64), ("c4-mini", 32)])
+def test_spmm_backward_is_transpose_spmm_and_sddmm(name, F):
+    adj = datasets.config_graph(name)
+    n_rows, n_cols = adj.shape
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((n_cols, F), dtype=np.float32)
+    dout = rng.standard_normal((n_rows, F), dtype=np.float32)
+    grad = VanillaSpMMGradhip(adj)
+    grad.build([placeholder(x.shape)])
+    dx, da = grad.run([nd.array(x, grad.ctx), nd.array(dout, grad.ctx)])
+    dx, da = dx.asnumpy(), da.asnumpy()
+    t = adj.T.tocsr()
+    assert np.array_equal(dx, ref.spmm_csr_x86(t.indptr, t.indices, t.data, dout))        # bit-exact on A^T
+    np.testing.assert_allclose(dx, adj.T.astype(np.float64).dot(dout.astype(np.float64)), rtol=1e-4, atol=2e-3)
+    coo = adj.tocoo()
+    np.testing.assert_allclose(da, ref.sddmm_f64(coo.row, coo.col, x, dout), rtol=RTOL, atol=ATOL)
+    # the defining identity of a gradient: <A x, dOut> = <x, A^T dOut> = sum_e vals[e] * dA[e]
+    lhs = float((adj.astype(np.float64).dot(x.astype(np.float64)) * dout).sum())
+    assert abs(lhs - float((x.astype(np.float64) * dx).sum())) <= 1e-6 * abs(lhs) + 1e-2
+    assert abs(lhs - float((adj.data.astype(np.float64) * da).sum())) <= 1e-6 * abs(lhs) + 1e-2

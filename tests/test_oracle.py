@@ -262,3 +262,86 @@ def test_softmax_weights_sum_to_one_per_row_and_head():
     w = datasets.softmax_edge_weights(adj, 8)
     sums = np.add.reduceat(w.astype(np.float64), adj.indptr[:-1][np.diff(adj.indptr) > 0], axis=0)
     np.testing.assert_allclose(sums, 1.0, rtol=0, atol=1e-5)
+
+
+# ---------------------------------------------------------------- DDS nest: per-block sums, then their sum
+def test_dds_adds_block_sums_not_terms():
+    """One row, columns [0,1 | 2,3] in two blocks, values 1e8, 1, -1e8, 1 (features all one).  Term by term the
+    float32 sum is 1 (fgref_spmm_csr_x86); block by block it is (1e8 + 1) + (-1e8 + 1) = 1e8 + (-1e8) = 0,
+    which is what the reference's DDS nest computes (op/vanilla_spmm.py:201-218)."""
+    adj = scipy.sparse.csr_matrix((np.array([1e8, 1, -1e8, 1], np.float32), np.arange(4, dtype=np.int32),
+                                   np.array([0, 4], np.int32)), shape=(1, 4))
+    feat = np.ones((4, 2), np.float32)
+    assert np.all(ref.spmm_csr_x86(adj.indptr, adj.indices, adj.data, feat) == 1.0)
+    s1_pos, s1_idx, vals = util_convert_csr_to_dds(adj, 2)
+    assert np.all(ref.spmm_dds_x86(s1_pos, s1_idx, vals, feat, 1, 2) == 0.0)
+
+
+# ---------------------------------------------------------------- generalised message / reduce / edge functions
+def _rows_with_edges(adj):
+    return np.flatnonzero(np.diff(adj.indptr) > 0)
+
+
+@pytest.mark.parametrize("msg", ["mul", "add", "sub", "div", "copy_u"])
+@pytest.mark.parametrize("reduce", ["sum", "max", "min", "mean"])
+def test_generalised_spmm_against_numpy_reduceat(msg, reduce):
+    adj, feat = _int_case(seed=3)
+    adj.data = np.random.default_rng(4).choice(np.array([1, 2, 4], np.float32), adj.nnz)   # exact quotients too
+    out = ref.spmm_general(adj.indptr, adj.indices, adj.data, feat, msg, reduce)
+    u, e = feat[adj.indices].astype(np.float64), adj.data.astype(np.float64)[:, None]
+    terms = {"mul": u * e, "add": u + e, "sub": u - e, "div": u / e, "copy_u": u}[msg]
+    rows = _rows_with_edges(adj)
+    starts = adj.indptr[rows]
+    fold = {"sum": np.add, "mean": np.add, "max": np.maximum, "min": np.minimum}[reduce].reduceat(terms, starts, axis=0)
+    if reduce == "mean":
+        fold = fold / np.diff(adj.indptr)[rows][:, None]
+    want = np.zeros((adj.shape[0], feat.shape[1]))
+    want[rows] = fold
+    if reduce == "mean":
+        np.testing.assert_allclose(out, want, rtol=1e-6, atol=0)       # one rounded division of an exact sum
+    else:
+        assert np.array_equal(out, want.astype(np.float32))            # integers and dyadic quotients: exact
+    assert np.all(out[np.diff(adj.indptr) == 0] == 0)                  # rows without edges give 0 under every reducer
+
+
+def test_generalised_spmm_mul_sum_is_the_vanilla_nest(adj_127x255):
+    adj = adj_127x255
+    feat = np.random.default_rng(5).standard_normal((adj.shape[1], 40), dtype=np.float32)
+    assert np.array_equal(ref.spmm_general(adj.indptr, adj.indices, adj.data, feat, "mul", "sum"),
+                          ref.spmm_csr_x86(adj.indptr, adj.indices, adj.data, feat))
+    # float operands: max / min pick an existing term exactly; sum stays within rounding of float64
+    for msg in ("add", "div"):
+        u, e = feat[adj.indices], adj.data[:, None] + np.float32(0.5)
+        terms = (u + e) if msg == "add" else (u / e)
+        rows = _rows_with_edges(adj)
+        got = ref.spmm_general(adj.indptr, adj.indices, adj.data + np.float32(0.5), feat, msg, "max")
+        assert np.array_equal(got[rows], np.maximum.reduceat(terms, adj.indptr[rows], axis=0))
+
+
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
+def test_generalised_sddmm_against_numpy(op):
+    coo = reference_test_matrix("coo", seed=2)
+    rng = np.random.default_rng(6)
+    src = rng.standard_normal((coo.shape[1], 24), dtype=np.float32)
+    dst = rng.standard_normal((coo.shape[0], 24), dtype=np.float32) + np.float32(3.0)
+    a, b = src[coo.col], dst[coo.row]
+    want = {"add": a + b, "sub": a - b, "mul": a * b, "div": a / b}[op]        # one rounded operation each
+    assert np.array_equal(ref.sddmm_general(coo.row, coo.col, src, dst, op), want)
+
+
+def test_edge_softmax_against_scipy_and_its_invariants():
+    import scipy.special
+    adj = datasets.config_graph("c4-mini")
+    H = 4
+    scores = (np.random.default_rng(7).standard_normal((adj.nnz, H)) * 5).astype(np.float32)
+    out = ref.edge_softmax(adj.indptr, scores)
+    for r in (0, 1, 17, 4242, adj.shape[0] - 1):
+        sl = slice(adj.indptr[r], adj.indptr[r + 1])
+        np.testing.assert_allclose(out[sl], scipy.special.softmax(scores[sl].astype(np.float64), axis=0), rtol=1e-6)
+    rows = _rows_with_edges(adj)
+    np.testing.assert_allclose(np.add.reduceat(out.astype(np.float64), adj.indptr[rows], axis=0), 1.0, atol=1e-5)
+    shifted = ref.edge_softmax(adj.indptr, scores + np.float32(8.0))          # shift invariance (8 is exact to add)
+    np.testing.assert_allclose(shifted, out, rtol=1e-5, atol=1e-9)
+    uniform = ref.edge_softmax(adj.indptr, np.zeros((adj.nnz, H), np.float32))
+    deg = np.repeat(np.diff(adj.indptr), np.diff(adj.indptr))
+    np.testing.assert_allclose(uniform, (1.0 / deg)[:, None].repeat(H, 1), rtol=1e-6)
