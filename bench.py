@@ -105,7 +105,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--feat-len", type=int, default=64, help="feature length of the timed step")
     ap.add_argument("--graph", default="c2", help="named synthetic configuration (featgraph_amd.datasets.CONFIGS)")
-    ap.add_argument("--only", choices=["all", "spmm", "sddmm", "copy", "mh_sddmm", "mh_spmm", "gather_probe"],
+    ap.add_argument("--only", choices=["all", "spmm", "sddmm", "copy", "mh_sddmm", "mh_spmm", "mh_sddmm_softmax",
+                                       "gather_probe"],
                     default="all",
                     help="spmm / sddmm / copy / gather_probe: run just that kernel (for profiler runs), no sweep, no "
                          "CPU leg; mh_sddmm / mh_spmm: the multi-head operators (8 heads of --feat-len floats, use "
@@ -121,7 +122,8 @@ def main():
     import numpy as np
     import torch
     from featgraph_amd import _lib, datasets, nd, placeholder
-    from featgraph_amd.module import MultiHeadSDDMMhip, MultiHeadSpMMhip, VanillaSDDMMhip, VanillaSpMMhip
+    from featgraph_amd.module import (EdgeSoftmaxhip, MultiHeadSDDMMhip, MultiHeadSDDMMSoftmaxhip, MultiHeadSpMMhip,
+                                      VanillaSDDMMhip, VanillaSpMMhip)
 
     L = _lib.lib()  # fail now if the HIP library is missing
     if not torch.cuda.is_available():
@@ -191,10 +193,12 @@ def main():
         H = MH_HEADS
         n_r, n_c, e = graph_adj.shape[0], graph_adj.shape[1], graph_adj.nnz
         row = {"op": kind, "H": H, "D": D}
-        if kind == "mh_sddmm":
+        if kind in ("mh_sddmm", "mh_sddmm_softmax"):
             coo = graph_adj.tocoo()
-            op = MultiHeadSDDMMhip(coo)
+            op = MultiHeadSDDMMhip(coo) if kind == "mh_sddmm" else MultiHeadSDDMMSoftmaxhip(coo)
             src, dst = device_normal((n_c, H, D), 11 + D), device_normal((n_r, H, D), 12 + D)
+            if kind == "mh_sddmm_softmax":
+                src *= 0.25                      # scores of magnitude ~ sqrt(D) / 4: weights that are not one-hot
             op.build([placeholder((n_c, H, D)), placeholder((n_r, H, D))], {}, {})
             ins = [src, dst]
             b, b_min = mh_sddmm_alg_bytes(e, H, D), 8 * e + 4 * H * e + 4 * H * D * (n_r + n_c)
@@ -228,12 +232,20 @@ def main():
                     want = ref.sddmm_mh(coo.row[sl], coo.col[sl], s_h, d_h)
                     ok = ok and bool(np.all(np.abs(out[sl] - want) <= ATOL + RTOL * np.abs(want)))
                 row["parity"] = {"within_rtol1e-5_atol1e-4_of_cpu_checker": ok, "edges_checked": 2 * m}
+            elif kind == "mh_sddmm_softmax":
+                # the first rows' edges: scores by the CPU checker, softmax in float64, against the fused kernel
+                n_check = int(np.searchsorted(graph_adj.indptr, 3_000_000))
+                m = int(graph_adj.indptr[n_check])
+                scores = ref.sddmm_mh(coo.row[:m], coo.col[:m], src.cpu().numpy(), dst.cpu().numpy())
+                want = ref.edge_softmax(graph_adj.indptr[:n_check + 1], scores)
+                ok = bool(np.all(np.abs(out[:m] - want) <= 1e-6 + 1e-4 * np.abs(want)))
+                row["parity"] = {"within_rtol1e-4_atol1e-6_of_cpu_checker": ok, "edges_checked": m}
             else:
                 want = ref.spmm_mh(graph_adj.indptr, graph_adj.indices, w.cpu().numpy(), src.cpu().numpy())
                 row["parity"] = {"bit_exact_vs_cpu_checker": bool(np.array_equal(out, want))}
         return row
 
-    if args.only in ("mh_sddmm", "mh_spmm"):
+    if args.only in ("mh_sddmm", "mh_spmm", "mh_sddmm_softmax"):
         row = mh_case(args.only, adj, F, args.steps, args.warmup, False)
         row.update({"kernel": args.only, "graph": args.graph})
         print(json.dumps(row))
@@ -414,6 +426,21 @@ def main():
             torch.cuda.empty_cache()
             log("mh_sddmm D=%d: %.3f ms (%.2f of the HBM roofline by algorithmic bytes)" % (
                 D, mh[-1]["ms"], mh[-1]["frac"]))
+        # the GAT chain between them: scores + edge softmax in one kernel, against the two operators run
+        # one after the other (multi-head SDDMM, then the softmax over its [nnz, 8] output)
+        for D in MH_HEAD_LENS:
+            mh.append(mh_case("mh_sddmm_softmax", big, D, 5, 1, check))
+            torch.cuda.empty_cache()
+            log("mh_sddmm_softmax (fused) D=%d: %.3f ms" % (D, mh[-1]["ms"]))
+        soft = EdgeSoftmaxhip(big)
+        soft.build([placeholder((big.nnz, MH_HEADS))], {}, {})
+        scores = device_normal((big.nnz, MH_HEADS), 5)
+        soft_ms = timed(lambda: soft.run([scores]), 5, 1)
+        mh.append({"op": "edge_softmax", "H": MH_HEADS, "ms": soft_ms,
+                   "note": "standalone pass over [nnz, 8] scores: what the fused operator saves on top of the "
+                           "scores' round trip"})
+        del soft, scores
+        torch.cuda.empty_cache()
         mh.append(mh_case("mh_spmm", big, 64, 5, 1, check))
         log("mh_spmm D=64: %.3f ms (%.2f of the HBM roofline by algorithmic bytes)" % (mh[-1]["ms"], mh[-1]["frac"]))
         result["multi_head"] = {"graph": "c4: %d vertices, %d edges" % (big.shape[0], big.nnz), "rows": mh,

@@ -746,6 +746,32 @@ int fg_sddmm_coo_plan_f32(const fg_sddmm_plan *plan, const float *src, const flo
                                   plan->n_rows * int64_t{D} * 4, static_cast<hipStream_t>(stream));
 }
 
+int fg_edge_softmax_csr_f32(int64_t n_rows, const int32_t *indptr, const float *scores, float *out, int32_t H,
+                            void *stream) {
+  if (n_rows < 0 || n_rows >= 0x7fffffffLL) return fg::fail(FG_EINVAL, "n_rows = %lld is out of range", (long long)n_rows);
+  if (H < 1 || H > (1 << 20)) return fg::fail(FG_EINVAL, "H = %d is out of range", H);
+  if (n_rows == 0) return FG_OK;
+  if (!indptr || !scores || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
+  return fg::edge_softmax_launch(indptr, scores, out, static_cast<int32_t>(n_rows), H, static_cast<hipStream_t>(stream));
+}
+
+int fg_sddmm_softmax_plan_f32(const fg_sddmm_plan *plan, const float *src, const float *dst, float *out, int32_t H,
+                              int32_t D, void *stream) {
+  if (!plan) return fg::fail(FG_EINVAL, "plan is null");
+  if (int rc = check_heads(H, D)) return rc;
+  if (plan->nnz == 0) return FG_OK;
+  if (int rc = check_device(plan->device)) return rc;
+  if (!src || !dst || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
+  if (!plan->indptr || !plan->rows)
+    return fg::fail(FG_EUNSUPPORTED, "edge softmax needs a row-sorted edge list (each destination row's edges consecutive)");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int32_t n = static_cast<int32_t>(plan->n_rows);
+  if (fg::sddmm_softmax_fused_applies(src, dst, H, D))
+    return fg::sddmm_softmax_launch(plan->rows->row_order, plan->indptr, plan->col, src, dst, out, n, H, D, st);
+  if (int rc = fg_sddmm_coo_plan_f32(plan, src, dst, out, H, D, stream)) return rc;
+  return fg::edge_softmax_launch(plan->indptr, out, out, n, H, st);
+}
+
 int fg_sddmm_plan_describe(const fg_sddmm_plan *plan, int32_t H, int32_t D, char *buf, int64_t cap) {
   if (!plan) return fg::fail(FG_EINVAL, "plan is null");
   if (!buf || cap <= 0) return fg::fail(FG_EINVAL, "no room for the description");

@@ -152,6 +152,13 @@ int spmm_general_launch(const int32_t *row_order, const int32_t *seg_lo, const i
 int sddmm_elementwise_launch(const int32_t *row, const int32_t *col, const float *src, const float *dst, float *out,
                              int64_t nnz, int32_t F, int op, hipStream_t stream);
 
+// Edge softmax over CSR rows, alone and fused into multi-head SDDMM (softmax.hip).
+int edge_softmax_launch(const int32_t *indptr, const float *scores, float *out, int32_t n_rows, int32_t H,
+                        hipStream_t stream);
+bool sddmm_softmax_fused_applies(const float *src, const float *dst, int32_t H, int32_t D);
+int sddmm_softmax_launch(const int32_t *row_order, const int32_t *indptr, const int32_t *indices, const float *src,
+                         const float *dst, float *out, int32_t n_rows, int32_t H, int32_t D, hipStream_t stream);
+
 inline bool aligned_to(const void *p, uintptr_t bytes) { return (reinterpret_cast<uintptr_t>(p) & (bytes - 1)) == 0; }
 
 inline int pow2_ceil(int x) {

@@ -1,3 +1,4 @@
 from .sddmm import VanillaSDDMMhip, MultiHeadSDDMMhip
 from .spmm import VanillaSpMMhip, MultiHeadSpMMhip
 from .general import GeneralizedSpMMhip, GeneralizedSDDMMhip, VanillaSpMMGradhip
+from .softmax import EdgeSoftmaxhip, MultiHeadSDDMMSoftmaxhip

@@ -215,6 +215,33 @@ FG_API int fg_sddmm_coo_plan_f32(const fg_sddmm_plan *plan, const float *src, co
 FG_API int fg_sddmm_plan_describe(const fg_sddmm_plan *plan, int32_t H, int32_t D, char *buf, int64_t cap);
 
 /*
+ * Edge softmax (no counterpart in the reference; the step between the scores of
+ * multi-head SDDMM and the weights of multi-head SpMM in a GAT-style layer).
+ * The edge list is the CSR one: row r's edges are [indptr[r], indptr[r+1]).
+ * out[e, h] = exp(scores[e, h] - max) / sum over the row's edges of
+ * exp(scores[e', h] - max), max taken over the same edges, per head.  scores
+ * and out are [nnz, H] and may be the same buffer.  Scores must be finite.
+ */
+FG_API int fg_edge_softmax_csr_f32(int64_t n_rows, const int32_t *indptr, const float *scores, float *out, int32_t H,
+                                   void *stream);
+/*
+ * fg_sddmm_coo_mh_f32 followed by fg_edge_softmax_csr_f32, on the plan's edge
+ * list, which must be row-sorted (FG_EUNSUPPORTED otherwise):
+ * out[e, h] = softmax over the edges of row[e] of sum_d src[col[e], h, d] * dst[row[e], h, d].
+ * When a vertex row (H * D floats) is one or two runs of 64 loads of 1, 2 or 4
+ * floats and a head spans 4, 8 or 16 of a run's lanes (H = 8 with D in {8, 16,
+ * 32, 64}; H = 4 with D in {16, 32, 64}; H = 16 with D in {4, 8, 16, 32}; ...)
+ * one fused kernel computes a destination row's scores, keeps their running
+ * maximum and sum, and normalises them in place, so the raw scores never
+ * travel through a second kernel; other shapes run the two kernels one after
+ * the other.  Float32
+ * throughout; agrees with the float64 softmax of the float32 scores within
+ * rtol 1e-5.
+ */
+FG_API int fg_sddmm_softmax_plan_f32(const fg_sddmm_plan *plan, const float *src, const float *dst, float *out,
+                                     int32_t H, int32_t D, void *stream);
+
+/*
  * Multi-head SDDMM (no counterpart in the reference; the edge function of
  * op/vanilla_sddmm.py:47 per head): Out[e, h] = sum_d src[col[e], h, d] * dst[row[e], h, d].
  * src [n_cols, H, D], dst [n_rows, H, D], out [nnz, H].  H = 1 gives

@@ -7,7 +7,8 @@ import numpy as np
 import pytest
 
 from featgraph_amd import datasets, nd, placeholder
-from featgraph_amd.module import MultiHeadSDDMMhip, MultiHeadSpMMhip, VanillaSDDMMhip, VanillaSpMMhip
+from featgraph_amd.module import (MultiHeadSDDMMhip, MultiHeadSDDMMSoftmaxhip, MultiHeadSpMMhip, VanillaSDDMMhip,
+                                  VanillaSpMMhip)
 from oracle import ref
 
 pytestmark = pytest.mark.gpu
@@ -209,6 +210,31 @@ def test_c4_multihead_sddmm_longer_heads(c4, D):
     del src_dev, dst_dev
     assert out.shape == (coo.nnz, H)
     np.testing.assert_allclose(out, ref.sddmm_mh(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("D", [16, 64])
+def test_c4_fused_scores_and_softmax(c4, D):
+    """The fused score + softmax kernel on the whole 2.45M-vertex graph (hub rows of 20,000 edges included),
+    against the CPU checker's scores normalised in float64."""
+    adj = c4
+    coo = adj.tocoo()
+    n, H = adj.shape[0], 8
+    _say("fused multi-head scores + softmax c4 H=8 D=%d through MultiHeadSDDMMSoftmaxhip" % D)
+    module = MultiHeadSDDMMSoftmaxhip(adj)
+    ph = [placeholder((n, H, D)), placeholder((n, H, D))]
+    assert "fused" in module.lower_to_ir(ph, {}, {})
+    module.build(ph, {}, {})
+    src_dev, src = _device_normal((n, H, D), 600 + D, module.ctx)
+    dst_dev, dst = _device_normal((n, H, D), 700 + D, module.ctx)
+    src_dev *= 0.25
+    src *= np.float32(0.25)
+    out = module.run([src_dev, dst_dev]).asnumpy()
+    del src_dev, dst_dev
+    want = ref.edge_softmax(adj.indptr, ref.sddmm_mh(coo.row, coo.col, src, dst))
+    np.testing.assert_allclose(out, want, rtol=1e-4, atol=1e-6)
+    rows = np.flatnonzero(np.diff(adj.indptr) > 0)
+    sums = np.add.reduceat(out.astype(np.float64), adj.indptr[rows].astype(np.int64), axis=0)
+    np.testing.assert_allclose(sums, 1.0, atol=1e-4)
 
 
 def test_benchmark_commands_run_on_a_small_graph(tmp_path, capsys):

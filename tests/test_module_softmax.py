@@ -1,0 +1,110 @@
+"""GPU parity of the edge softmax and of the fused multi-head score + softmax operator, through the module layer
+and the C ABI.  The checker computes the softmax in float64 (oracle/featgraph_ref.c: fgref_edge_softmax); the
+kernels work in float32, so the bar is a tolerance: rtol 1e-5 with atol 1e-7 on weights that lie in (0, 1]."""
+import numpy as np
+import pytest
+import scipy.sparse
+
+from featgraph_amd import _lib, datasets, nd, placeholder
+from featgraph_amd.module import EdgeSoftmaxhip, MultiHeadSDDMMhip, MultiHeadSDDMMSoftmaxhip, MultiHeadSpMMhip
+from oracle import ref
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-5, 1e-7
+
+
+def _softmax_module(adj, scores):
+    module = EdgeSoftmaxhip(adj)
+    module.build([placeholder(scores.shape)], {}, {})
+    return module.run([nd.array(scores, module.ctx)]).asnumpy()
+
+
+@pytest.mark.parametrize("H", [1, 2, 4, 8, 16, 64, 3, 5, 100])
+def test_edge_softmax_matches_the_float64_checker(H):
+    adj = datasets.config_graph("c4-mini")              # degrees 1 .. 2,000, mean 25
+    scores = (np.random.default_rng(H).standard_normal((adj.nnz, H)) * 4).astype(np.float32)
+    out = _softmax_module(adj, scores)
+    np.testing.assert_allclose(out, ref.edge_softmax(adj.indptr, scores), rtol=RTOL, atol=ATOL)
+    rows = np.flatnonzero(np.diff(adj.indptr) > 0)
+    np.testing.assert_allclose(np.add.reduceat(out.astype(np.float64), adj.indptr[rows], axis=0), 1.0, atol=1e-5)
+
+
+def test_edge_softmax_with_empty_rows_single_edges_and_large_scores():
+    indptr = np.array([0, 0, 1, 1, 4, 4, 300], dtype=np.int32)       # rows 0, 2, 4 empty; row 1 has one edge
+    n, nnz = len(indptr) - 1, int(indptr[-1])
+    adj = scipy.sparse.csr_matrix((np.ones(nnz, np.float32), np.zeros(nnz, np.int32), indptr), shape=(n, 1))
+    scores = (np.random.default_rng(1).standard_normal((nnz, 8)) * 30 + 80).astype(np.float32)   # exp(80) overflows float32
+    out = _softmax_module(adj, scores)
+    assert np.all(np.isfinite(out)) and np.all(out[0] == 1.0)        # a single edge takes all the weight
+    np.testing.assert_allclose(out, ref.edge_softmax(indptr, scores), rtol=RTOL, atol=ATOL)
+
+
+def test_edge_softmax_in_place_through_the_c_abi():
+    import torch
+    adj = datasets.config_graph("c4-mini")
+    scores = np.random.default_rng(3).standard_normal((adj.nnz, 8)).astype(np.float32)
+    dev = torch.device("cuda", 0)
+    buf = torch.from_numpy(scores).to(dev)
+    indptr = torch.from_numpy(adj.indptr.astype(np.int32)).to(dev)
+    _lib.check(_lib.lib().fg_edge_softmax_csr_f32(adj.shape[0], indptr.data_ptr(), buf.data_ptr(), buf.data_ptr(), 8,
+                                                  torch.cuda.current_stream(dev).cuda_stream))
+    np.testing.assert_allclose(buf.cpu().numpy(), ref.edge_softmax(adj.indptr, scores), rtol=RTOL, atol=ATOL)
+
+
+def _fused(adj, src, dst):
+    module = MultiHeadSDDMMSoftmaxhip(adj)
+    ph = [placeholder(src.shape), placeholder(dst.shape)]
+    module.build(ph, {}, {})
+    module.out_tvm.tensor.fill_(-5.0)
+    return module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy(), module.lower_to_ir(ph, {}, {})
+
+
+@pytest.mark.parametrize("H,D,fused", [(8, 64, True), (8, 32, True), (8, 16, True), (8, 8, True), (4, 64, True),
+                                       (4, 128, False), (16, 4, True), (16, 32, True), (32, 8, True), (4, 16, True),
+                                       (8, 24, False),
+                                       (2, 32, False), (3, 5, False), (1, 64, False)])
+def test_fused_scores_and_softmax(H, D, fused):
+    adj = datasets.config_graph("c4-mini")
+    coo = adj.tocoo()
+    src, dst = datasets.sddmm_operands(coo, (H, D))
+    src *= np.float32(0.5)                                # keeps the scores in a range where the weights are not one-hot
+    out, text = _fused(adj, src, dst)
+    assert ("fused" in text) == fused
+    assert out.shape == (coo.nnz, H)
+    scores64 = np.einsum("ehd,ehd->eh", src[coo.col].astype(np.float64), dst[coo.row].astype(np.float64))
+    want = ref.edge_softmax(adj.indptr, scores64.astype(np.float32))
+    # the kernel's float32 scores differ from the rounded float64 ones by a few ulps of a value of magnitude ~10,
+    # which the exponential turns into a relative error of that absolute size: ~1e-5
+    np.testing.assert_allclose(out, want, rtol=5e-5, atol=1e-7)
+    rows = np.flatnonzero(np.diff(adj.indptr) > 0)
+    np.testing.assert_allclose(np.add.reduceat(out.astype(np.float64), adj.indptr[rows], axis=0), 1.0, atol=1e-5)
+
+
+def test_fused_equals_the_two_operators_run_separately():
+    adj = datasets.config_graph("c4-mini")
+    coo = adj.tocoo()
+    H, D = 8, 64
+    src, dst = datasets.sddmm_operands(coo, (H, D))
+    src *= np.float32(0.25)
+    fused, _ = _fused(adj, src, dst)
+    sddmm = MultiHeadSDDMMhip(coo)
+    sddmm.build([placeholder(src.shape), placeholder(dst.shape)], {}, {})
+    scores = sddmm.run([nd.array(src, sddmm.ctx), nd.array(dst, sddmm.ctx)]).asnumpy()
+    np.testing.assert_allclose(fused, ref.edge_softmax(adj.indptr, scores), rtol=5e-5, atol=1e-7)
+    # ... and the weights drive multi-head SpMM: every output row is a convex combination of its neighbours' rows
+    feat = datasets.spmm_operands(adj, (H, D))
+    spmm = MultiHeadSpMMhip(adj)
+    spmm.build([placeholder(feat.shape), placeholder(fused.shape)], {}, {})
+    out = spmm.run([nd.array(feat, spmm.ctx), nd.array(fused, spmm.ctx)]).asnumpy()
+    assert np.array_equal(out, ref.spmm_mh(adj.indptr, adj.indices, fused, feat))
+    ones = spmm.run([nd.array(np.ones_like(feat), spmm.ctx), nd.array(fused, spmm.ctx)]).asnumpy()
+    np.testing.assert_allclose(ones[np.diff(adj.indptr) > 0], 1.0, atol=1e-4)
+
+
+def test_fused_operator_rejects_an_unsorted_edge_list():
+    adj = datasets.config_graph("c1").tocoo()
+    perm = np.random.default_rng(0).permutation(adj.nnz)
+    shuffled = scipy.sparse.coo_matrix((adj.data[perm], (adj.row[perm], adj.col[perm])), shape=adj.shape)
+    with pytest.raises(ValueError):
+        MultiHeadSDDMMSoftmaxhip(shuffled)
