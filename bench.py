@@ -164,6 +164,18 @@ def main():
         return {"ms": ms * n_gathers / issued, "tile": tile, "band_rows": band, "gathers_per_tile": n_gathers,
                 "row_TBps": n_gathers * F * 4 / (ms * n_gathers / issued) / 1e9}
 
+    def rows_probe(feat_t, n_gathers, steps=3):
+        """Milliseconds that n_gathers random whole-row gathers from feat_t take (rows of 128 .. 1024 floats)."""
+        n, row_floats = feat_t.shape[0], int(feat_t[0].numel())
+        issued = L.fg_probe_gather_rows_count(row_floats, n_gathers)
+        if issued <= 0:
+            return None
+        ms = timed(lambda: _lib.check(L.fg_probe_gather_rows_f32(feat_t.data_ptr(), n, row_floats, n_gathers,
+                                                                 sink.data_ptr(), stream.cuda_stream)), steps, 1)
+        ms = ms * n_gathers / issued
+        return {"ms": ms, "row_bytes": row_floats * 4, "gathers": n_gathers,
+                "row_TBps": n_gathers * row_floats * 4 / ms / 1e9}
+
     if args.only == "copy":
         # plain device copy of known size: the yardstick the byte counters are scaled with
         n = 1 << 28
@@ -218,6 +230,10 @@ def main():
             ins = [src, w]
             b, b_min = mh_spmm_alg_bytes(e, n_r, H, D), 4 * e + 4 * H * e + 4 * (n_r + 1) + 4 * H * D * (n_r + n_c)
         ms = timed(lambda: op.run(ins), steps, warmup)
+        p = rows_probe(src, e)
+        if p:
+            row.update({"gather_ceiling_ms": p["ms"], "gather_ceiling_row_TBps": p["row_TBps"],
+                        "frac_of_gather_ceiling": p["ms"] / ms})
         row.update({"ms": ms, "GFLOPs": 2.0 * e * H * D / ms / 1e6, "alg_GBps": b / ms / 1e6,
                     "frac": b / ms / 1e6 / HBM_PEAK_GBPS, "hbm_frac_compulsory": b_min / ms / 1e6 / HBM_PEAK_GBPS,
                     "algorithmic_bytes": b, "compulsory_bytes": b_min})
@@ -287,7 +303,7 @@ def main():
     achieved = alg / ms / 1e6
     gpu_out = spmm.out_tvm.asnumpy() if args.only == "all" else None
     traffic, traffic_source = committed_traffic("spmm", args.graph, F)
-    probe = gather_probe(feat.tensor, nnz)
+    probe = gather_probe(feat.tensor, nnz) if args.only == "all" else None
     roofline = {
         "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
         "traffic": traffic, "traffic_source": traffic_source,

@@ -52,6 +52,7 @@ struct fg_spmm_plan {
   // what the bounds table is built from: block width (0: default), blocks on / off / automatic (1 / 0 / -1),
   // and the nonzeros per (row, block) below which automatic mode keeps whole rows
   int32_t want_block_cols;
+  int32_t default_block_cols;  // the library's own pass width for 64-float tiles when nobody sized the blocks
   int want_blocked;
   double min_per_segment;
   // Records of the several-rows-per-wave kernel: whole rows, and column-block passes for its tiles of 16, 32
@@ -74,8 +75,8 @@ struct fg_sddmm_plan {
 };
 
 static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr, const int32_t *indices,
-                           int32_t num_col_partitions, int32_t want_block_cols, int want_blocked,
-                           double min_per_segment, bool with_multi, fg_spmm_plan **plan);
+                           int32_t num_col_partitions, int32_t want_block_cols, int32_t default_block_cols,
+                           int want_blocked, double min_per_segment, bool with_multi, fg_spmm_plan **plan);
 
 namespace {
 
@@ -142,6 +143,14 @@ int check_device(int plan_device) {
   return FG_OK;
 }
 
+// Default pass widths, in columns, for tiles of 64 floats (narrower tiles take proportionally more columns, so the
+// band of the feature matrix that a pass gathers from keeps its size).  One XCD's L2 is 4 MB = 16384 such rows.
+// SDDMM is fastest with the band at that size; SpMM, which pays a read and a write of every row's partial sum
+// per pass, with a band a quarter larger and correspondingly fewer passes (232,965-vertex graph, 64 floats:
+// 12 passes of 19,414 columns 1.86 ms, 15 of 15,532 1.95 ms, 9 of 25,885 1.98 ms).
+constexpr int32_t kSpmmBlockCols = 20480;
+constexpr int32_t kSddmmBlockCols = 16384;
+
 int check_heads(int32_t H, int32_t D) {
   if (H < 1 || D < 1) return fg::fail(FG_EINVAL, "H = %d and D = %d must both be positive", H, D);
   if (static_cast<int64_t>(H) * D > (1 << 20))
@@ -198,8 +207,7 @@ int multi_tile_index(int tile) { return tile == 16 ? 0 : tile == 32 ? 1 : 2; }
 int multi_merge(const fg_spmm_plan *plan, int tile) {
   if (plan->n_blocks < 2) return 1;
   if (plan->force_blocks || plan->want_block_cols > 0) return 1;
-  const int64_t m = (int64_t{4} << 20) / (tile * 4) / std::max(plan->block_cols, 1);
-  return static_cast<int>(std::min<int64_t>(std::max<int64_t>(m, 1), plan->n_blocks));
+  return std::min(64 / tile, plan->n_blocks);  // the table's blocks are sized for 64-float tiles
 }
 
 int multi_build(fg_spmm_plan *p) {
@@ -317,10 +325,12 @@ int sddmm_prepare(int64_t nnz, const int32_t *row, const int32_t *col, const flo
 // amortise re-reading its partial sum; otherwise the table holds whole rows.
 int build_bounds(fg_spmm_plan *p) {
   if (p->n_rows == 0) return FG_OK;
-  int64_t block_cols = p->want_block_cols > 0 ? p->want_block_cols : 16384;
+  int64_t block_cols = p->want_block_cols > 0 ? p->want_block_cols : p->default_block_cols;
   const int P = p->requested_partitions;
   if (P > 1) block_cols = std::max<int64_t>(1, (p->n_cols + P - 1) / P);  // util/adj_partitioning.py:42
   int64_t n_blocks = p->n_cols > 0 ? (p->n_cols + block_cols - 1) / block_cols : 1;
+  // the library's own blocks: as many as the default width asks for, all of the same width
+  if (P <= 1 && p->want_block_cols <= 0 && n_blocks > 1) block_cols = (p->n_cols + n_blocks - 1) / n_blocks;
   const double per_segment =
       n_blocks > 0 ? static_cast<double>(p->nnz) / (static_cast<double>(p->n_rows) * n_blocks) : 0.0;
   if (P == 1 || n_blocks < 2 || p->nnz == 0)
@@ -435,14 +445,14 @@ int fg_spmm_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32
 int fg_spmm_plan_create_partitioned(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr,
                                     const int32_t *indices, int32_t num_col_partitions, fg_spmm_plan **plan) {
   return row_plan_create(n_rows, n_cols, nnz, indptr, indices, num_col_partitions, fg::config().spmm_block_cols,
-                         fg::config().spmm_blocked, 8.0, true, plan);
+                         kSpmmBlockCols, fg::config().spmm_blocked, 8.0, true, plan);
 }
 
 // want_block_cols / want_blocked / min_per_segment: see fg_spmm_plan; with_multi: also build the records of the
 // several-rows-per-wave kernel.
 static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr, const int32_t *indices,
-                           int32_t num_col_partitions, int32_t want_block_cols, int want_blocked,
-                           double min_per_segment, bool with_multi, fg_spmm_plan **plan) {
+                           int32_t num_col_partitions, int32_t want_block_cols, int32_t default_block_cols,
+                           int want_blocked, double min_per_segment, bool with_multi, fg_spmm_plan **plan) {
   if (!plan) return fg::fail(FG_EINVAL, "plan output pointer is null");
   *plan = nullptr;
   if (num_col_partitions < 0)
@@ -492,6 +502,7 @@ static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const in
   p->requested_partitions = num_col_partitions;
   p->force_blocks = false;
   p->want_block_cols = want_block_cols;
+  p->default_block_cols = default_block_cols;
   p->want_blocked = want_blocked;
   p->min_per_segment = min_per_segment;
   p->max_degree = max_degree;
@@ -636,7 +647,8 @@ static int build_row_runs(fg_sddmm_plan *p, int32_t num_col_partitions) {
   // same block width as the re-ordered edge list (sddmm_blocked.hip); a run costs a wave a fixed amount of
   // work, so blocks need 8 edges per run on average (sparser lists keep whole rows and take the edge-list path)
   return row_plan_create(p->n_rows, p->n_cols, p->nnz, p->indptr, p->col, num_col_partitions,
-                         fg::config().sddmm_block_cols, fg::config().sddmm_blocked, 8.0, false, &p->rows);
+                         fg::config().sddmm_block_cols, kSddmmBlockCols, fg::config().sddmm_blocked, 8.0, false,
+                         &p->rows);
 }
 
 int fg_sddmm_plan_create(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,
@@ -704,8 +716,7 @@ static bool sddmm_use_blocks(const fg_sddmm_plan *plan, const float *src, const 
 static int sddmm_rows_merge(const fg_sddmm_plan *plan, int32_t D) {
   const fg_spmm_plan *r = plan->rows;
   if (plan->force_blocks || r->want_block_cols > 0 || r->n_blocks < 2) return 1;
-  const int64_t band_cols = (int64_t{4} << 20) / (fg::sddmm_rows_tile(D) * 4);
-  return static_cast<int>(std::max<int64_t>(1, band_cols / r->block_cols));
+  return 64 / fg::sddmm_rows_tile(D);  // the table's blocks are sized for 64-float tiles
 }
 
 static bool sddmm_use_row_runs(const fg_sddmm_plan *plan, const float *src, const float *dst, int32_t H, int32_t D) {

@@ -51,7 +51,90 @@ __global__ __launch_bounds__(fg::kBlockThreads) void probe_gather_kernel(const f
   if (acc.x + acc.y + acc.z + acc.w == __builtin_inff()) sink[0] = acc.x;
 }
 
+// Whole rows of `row_floats` floats (128, 256, or a multiple of 256) from anywhere in the matrix, addressed
+// in 64 bits: the pattern of the multi-head operators, whose feature matrices are far larger than any cache.
+// LPR lanes fetch one row with NV 16-byte loads each; 16 loads are in flight per lane.
+template <int LPR, int NV>
+__global__ __launch_bounds__(fg::kBlockThreads) void probe_rows_kernel(const float *feat, int64_t row_floats,
+                                                                       uint32_t n_rows, int iters, float *sink) {
+  constexpr int U = 16 / NV;
+  const int lane = threadIdx.x & (fg::kWaveSize - 1);
+  const int gl = lane & (LPR - 1), g = lane / LPR;
+  const uint32_t wave = blockIdx.x * fg::kWavesPerBlock + (threadIdx.x >> 6);
+  uint32_t s = wave * 2654435761u + static_cast<uint32_t>(g) * 40503u + 12345u;
+  float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  for (int it = 0; it < iters; ++it) {
+    float4 x[U][NV];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      s = s * 1664525u + 1013904223u;
+      const uint32_t r = (s >> 4) % n_rows;
+      const float *p = feat + static_cast<int64_t>(r) * row_floats + gl * 4;
+#pragma unroll
+      for (int k = 0; k < NV; ++k) x[u][k] = *reinterpret_cast<const float4 *>(p + k * 256);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int k = 0; k < NV; ++k) {
+        acc.x += x[u][k].x;
+        acc.y += x[u][k].y;
+        acc.z += x[u][k].z;
+        acc.w += x[u][k].w;
+      }
+  }
+  if (acc.x + acc.y + acc.z + acc.w == __builtin_inff()) sink[0] = acc.x;
+}
+
+// (lanes per row, loads per lane, rows per iteration of the grid) for a row length, or false.
+bool rows_shape(int32_t row_floats, int *lpr, int *nv, int64_t *per_iter) {
+  if (row_floats == 128)
+    *lpr = 32, *nv = 1;
+  else if (row_floats == 256)
+    *lpr = 64, *nv = 1;
+  else if (row_floats == 512)
+    *lpr = 64, *nv = 2;
+  else if (row_floats == 1024)
+    *lpr = 64, *nv = 4;
+  else
+    return false;
+  *per_iter = int64_t{kProbeBlocks} * fg::kWavesPerBlock * (fg::kWaveSize / *lpr) * (16 / *nv);
+  return true;
+}
+
 }  // namespace
+
+extern "C" int fg_probe_gather_rows_f32(const float *feat, int64_t n_rows, int32_t row_floats, int64_t n_gathers,
+                                        float *sink, void *stream) {
+  if (!feat || !sink) return fg::fail(FG_EINVAL, "feat or sink is null");
+  int lpr, nv;
+  int64_t per_iter;
+  if (!rows_shape(row_floats, &lpr, &nv, &per_iter))
+    return fg::fail(FG_EINVAL, "row_floats = %d is not one of 128, 256, 512, 1024", row_floats);
+  if (n_rows < 1 || n_rows > 0xffffffffLL || n_gathers < 0) return fg::fail(FG_EINVAL, "n_rows or n_gathers out of range");
+  if (!fg::aligned_to(feat, 16)) return fg::fail(FG_EINVAL, "feat must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int iters = static_cast<int>(std::max<int64_t>(1, (n_gathers + per_iter / 2) / per_iter));
+  const uint32_t n = static_cast<uint32_t>(n_rows);
+  const dim3 grid(kProbeBlocks), block(fg::kBlockThreads);
+  if (row_floats == 128)
+    probe_rows_kernel<32, 1><<<grid, block, 0, st>>>(feat, row_floats, n, iters, sink);
+  else if (row_floats == 256)
+    probe_rows_kernel<64, 1><<<grid, block, 0, st>>>(feat, row_floats, n, iters, sink);
+  else if (row_floats == 512)
+    probe_rows_kernel<64, 2><<<grid, block, 0, st>>>(feat, row_floats, n, iters, sink);
+  else
+    probe_rows_kernel<64, 4><<<grid, block, 0, st>>>(feat, row_floats, n, iters, sink);
+  FG_HIP_TRY(hipGetLastError());
+  return FG_OK;
+}
+
+extern "C" int64_t fg_probe_gather_rows_count(int32_t row_floats, int64_t n_gathers) {
+  int lpr, nv;
+  int64_t per_iter;
+  if (!rows_shape(row_floats, &lpr, &nv, &per_iter) || n_gathers < 0) return -1;
+  return std::max<int64_t>(1, (n_gathers + per_iter / 2) / per_iter) * per_iter;
+}
 
 extern "C" int fg_probe_gather_f32(const float *feat, int64_t n_rows, int32_t F, int32_t tile, int32_t band_rows,
                                    int64_t n_gathers, float *sink, void *stream) {

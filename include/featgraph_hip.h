@@ -60,11 +60,11 @@ FG_API const char *fg_last_error(void);
  * nnz, and stores on the device the row ids sorted by descending degree (ties
  * by ascending row id).  When the matrix is wide and dense enough for column
  * blocking to pay off and every row's column ids ascend, it also stores, per
- * block of 16384 columns, where that block starts inside every row (one device
- * pass over indices; (n_cols/16384 + 2) * n_rows int32), and for the default
+ * block of about 20000 columns (equal widths), where that block starts inside every row (one device
+ * pass over indices; (n_cols/20480 + 3) * n_rows int32), and for the default
  * kernel one 16-byte record {first nonzero, one past the last, row id} per row
  * and column-block pass, each pass sorted by descending run length (device
- * radix sorts; with blocks about (n_cols/16384) * 2 * n_rows records, else
+ * radix sorts; with blocks about (n_cols/20480) * 2 * n_rows records, else
  * n_rows).  The plan BORROWS indptr and indices: both must stay alive and
  * unchanged until fg_spmm_plan_destroy.
  */
@@ -273,6 +273,16 @@ FG_API int fg_check_indices(int64_t n, const int32_t *idx, int64_t bound, int64_
 FG_API int fg_probe_gather_f32(const float *feat, int64_t n_rows, int32_t F, int32_t tile, int32_t band_rows,
                                int64_t n_gathers, float *sink, void *stream);
 FG_API int64_t fg_probe_gather_count(int64_t n_rows, int32_t tile, int32_t band_rows, int64_t n_gathers);
+/*
+ * The same for the multi-head operators, whose feature matrices are far beyond
+ * any cache: about n_gathers whole rows of row_floats floats (128, 256, 512 or
+ * 1024) from random places of feat [n_rows, row_floats], 16-byte loads, 64-bit
+ * addressing, sixteen loads in flight per lane, one launch.  What it sustains
+ * is the rate at which this part's HBM serves random row gathers.
+ */
+FG_API int fg_probe_gather_rows_f32(const float *feat, int64_t n_rows, int32_t row_floats, int64_t n_gathers,
+                                    float *sink, void *stream);
+FG_API int64_t fg_probe_gather_rows_count(int32_t row_floats, int64_t n_gathers);
 
 /*
  * Launch-shape overrides for tuning and tests.  The store is process-global
