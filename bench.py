@@ -84,6 +84,16 @@ def committed_traffic(op, graph, F):
     return (float(m.group(1)), rel) if m else (None, None)
 
 
+def committed_traffic_mh(kind, D):
+    """The same for a multi-head operator on the 2.45M-vertex graph."""
+    rel = os.path.join("profiles", "multihead_c4_counters.txt")
+    path = os.path.join(ROOT, rel)
+    if not os.path.exists(path):
+        return None, None
+    m = re.search(r"^traffic_bytes_per_launch %s D=%d:\s*([0-9.eE+]+)" % (kind, D), open(path).read(), flags=re.M)
+    return (float(m.group(1)), rel) if m else (None, None)
+
+
 def cpu_model():
     try:
         for line in open("/proc/cpuinfo"):
@@ -234,6 +244,9 @@ def main():
         if p:
             row.update({"gather_ceiling_ms": p["ms"], "gather_ceiling_row_TBps": p["row_TBps"],
                         "frac_of_gather_ceiling": p["ms"] / ms})
+        tr, tr_src = committed_traffic_mh(kind, D) if graph_adj.shape[0] == 2449029 else (None, None)
+        if tr:
+            row.update({"traffic": tr, "traffic_source": tr_src, "hbm_frac_traffic": tr / ms / 1e6 / HBM_PEAK_GBPS})
         row.update({"ms": ms, "GFLOPs": 2.0 * e * H * D / ms / 1e6, "alg_GBps": b / ms / 1e6,
                     "frac": b / ms / 1e6 / HBM_PEAK_GBPS, "hbm_frac_compulsory": b_min / ms / 1e6 / HBM_PEAK_GBPS,
                     "algorithmic_bytes": b, "compulsory_bytes": b_min})
@@ -460,8 +473,12 @@ def main():
         mh.append(mh_case("mh_spmm", big, 64, 5, 1, check))
         log("mh_spmm D=64: %.3f ms (%.2f of the HBM roofline by algorithmic bytes)" % (mh[-1]["ms"], mh[-1]["frac"]))
         result["multi_head"] = {"graph": "c4: %d vertices, %d edges" % (big.shape[0], big.nnz), "rows": mh,
-                                "note": "5 GB of features and mean degree 25: nothing for a cache to reuse, so "
-                                        "here `frac` (algorithmic bytes / time / 8 TB/s) is an HBM fraction"}
+                                "note": "1.25 - 5 GB of features and mean degree 25: nearly every neighbour gather "
+                                        "goes to HBM.  `frac` is algorithmic bytes / time / 8 TB/s (above 1 for SDDMM "
+                                        "because consecutive edges share their Dst row, which caches serve); "
+                                        "hbm_frac_traffic is the committed rocprofv3 byte count of the operator / time "
+                                        "/ 8 TB/s; frac_of_gather_ceiling is the time of the same number of random "
+                                        "whole-row gathers and nothing else (fg_probe_gather_rows_f32) / time"}
         del big
         torch.cuda.empty_cache()
 
