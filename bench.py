@@ -160,7 +160,7 @@ def main():
 
     sink = torch.zeros(64, dtype=torch.float32, device=dev)
 
-    def gather_probe(feat_t, n_gathers, steps=5):
+    def gather_probe(feat_t, n_gathers, steps=5, warmup=3):
         """Milliseconds that the bare gather pattern takes for n_gathers row gathers per tile, with the tile width and
         band width of the operators (a 4 MB band: 16384 rows of a 64-float tile)."""
         n, F = feat_t.shape
@@ -170,7 +170,7 @@ def main():
         band = 16384 * (64 // tile)
         issued = L.fg_probe_gather_count(n, tile, band, n_gathers)
         ms = timed(lambda: _lib.check(L.fg_probe_gather_f32(feat_t.data_ptr(), n, F, tile, band, n_gathers,
-                                                            sink.data_ptr(), stream.cuda_stream)), steps, 1)
+                                                            sink.data_ptr(), stream.cuda_stream)), steps, warmup)
         return {"ms": ms * n_gathers / issued, "tile": tile, "band_rows": band, "gathers_per_tile": n_gathers,
                 "row_TBps": n_gathers * F * 4 / (ms * n_gathers / issued) / 1e9}
 
