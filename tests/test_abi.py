@@ -83,3 +83,29 @@ def test_sddmm_launch_description_is_host_only():
     assert "lanes/dot=4" in text and "H=8" in text
     assert _lib.lib().fg_sddmm_describe(1000, 1, 64, buf, len(buf)) == 0
     assert "lanes/dot=16" in buf.value.decode()
+
+
+def test_error_codes_of_the_later_entry_points_without_a_device():
+    L = _lib.lib()
+    # generalised operators: bad codes and null plans are rejected before anything touches a device
+    assert L.fg_spmm_csr_general_f32(None, None, None, None, 4, 0, 0, None) == -1
+    assert L.fg_sddmm_coo_general_f32(4, 8, 8, 8, 8, 8, 4, 7, None) == -1                # no such edge function
+    assert L.fg_sddmm_coo_general_f32(-1, 8, 8, 8, 8, 8, 4, 1, None) == -1
+    assert L.fg_sddmm_coo_general_f32(0, None, None, None, None, None, 4, 2, None) == 0  # empty edge list
+    # edge softmax
+    assert L.fg_edge_softmax_csr_f32(-1, None, None, None, 8, None) == -1
+    assert L.fg_edge_softmax_csr_f32(4, None, None, None, 8, None) == -1                 # null data
+    assert L.fg_edge_softmax_csr_f32(4, 8, 8, 8, 0, None) == -1                          # H = 0
+    assert L.fg_edge_softmax_csr_f32(0, None, None, None, 8, None) == 0
+    assert L.fg_sddmm_softmax_plan_f32(None, None, None, None, 8, 64, None) == -1
+    # allocation-free SpMM
+    assert L.fg_spmm_csr_noalloc_f32((1 << 20) + 1, 8, 0, 8, None, None, None, 8, 4, None) == -4
+    assert b"1048576" in L.fg_last_error()
+    assert L.fg_spmm_csr_noalloc_f32(4, 4, 0, 8, None, None, None, 8, 0, None) == -1     # F = 0
+    # gather probes
+    assert L.fg_probe_gather_f32(None, 4, 64, 64, 16384, 0, None, None) == -1
+    assert L.fg_probe_gather_f32(8, 4, 60, 64, 16384, 0, 8, None) == -1                  # F not a multiple of the tile
+    assert L.fg_probe_gather_count(4, 48, 16384, 10) == -1
+    assert L.fg_probe_gather_count(232965, 64, 16384, 114606755) >= 100_000_000
+    assert L.fg_probe_gather_rows_f32(8, 4, 100, 10, 8, None) == -1
+    assert L.fg_probe_gather_rows_count(512, 61948164) >= 60_000_000

@@ -56,3 +56,43 @@ def test_noalloc_spmm_rejects_what_it_cannot_hold():
     assert rc == -4 and b"exceeds" in L.fg_last_error()
     assert L.fg_spmm_csr_noalloc_f32(4, 4, 0, None, None, None, None, 8, 4, None) == -1   # null indptr
     assert L.fg_spmm_csr_noalloc_f32(0, 4, 0, 8, None, None, None, None, 4, None) == 0    # no rows: nothing to do
+
+
+def test_noalloc_spmm_replays_from_a_hip_graph():
+    """The entry point enqueues kernels only (its counters are cleared by a fill kernel, not a memset), so after one
+    eager call (which looks up the built-in array's address) it can be recorded into a HIP graph; every replay must
+    reproduce the eager result, also after the operands changed and with eager work between the replays."""
+    L = _lib.lib()
+    dev = torch.device("cuda", 0)
+    adj = datasets.config_graph("c2-mini")
+    n_rows, n_cols = adj.shape
+    F = 64
+    indptr = torch.from_numpy(adj.indptr.astype(np.int32)).to(dev)
+    indices = torch.from_numpy(adj.indices.astype(np.int32)).to(dev)
+    vals = torch.from_numpy(adj.data.astype(np.float32)).to(dev)
+    feat = torch.zeros((n_cols, F), dtype=torch.float32, device=dev)
+    out = torch.zeros((n_rows, F), dtype=torch.float32, device=dev)
+
+    def call():
+        _lib.check(L.fg_spmm_csr_noalloc_f32(n_rows, n_cols, adj.nnz, indptr.data_ptr(), indices.data_ptr(),
+                                             vals.data_ptr(), feat.data_ptr(), out.data_ptr(), F,
+                                             torch.cuda.current_stream(dev).cuda_stream))
+
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        call()                                        # outside the capture: first call on this device
+    torch.cuda.current_stream(dev).wait_stream(side)
+    torch.cuda.synchronize(dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    from oracle import ref
+    rng = np.random.default_rng(5)
+    for step in range(3):
+        x = rng.standard_normal((n_cols, F)).astype(np.float32)
+        feat.copy_(torch.from_numpy(x))
+        out.fill_(3.0)                                # eager work between the replays
+        graph.replay()
+        torch.cuda.synchronize(dev)
+        assert np.array_equal(out.cpu().numpy(), ref.spmm_csr_x86(adj.indptr, adj.indices, adj.data, x)), step
