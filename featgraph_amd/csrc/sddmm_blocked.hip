@@ -5,14 +5,14 @@
 // 232,965-vertex benchmark graph 28.6 GB per launch cross the L2 boundary at
 // 64 floats, and the kernel sits on that boundary's ~7.6 TB/s).  Here the plan
 // holds the edge list re-ordered by column block: first every edge whose column
-// id is below block_cols, then the next block, and inside a block the caller's
-// order (a stable sort).  One launch walks that list front to back; workgroups
+// id is below block_cols, then the next block, and inside a block by destination
+// row (a stable sort: equal keys keep the caller's order).  One launch walks
+// that list front to back; workgroups
 // are dispatched in list order, so at any moment the resident waves work on a
 // short window of the list, i.e. on one column block, whose Src rows
 // (block_cols x 64 floats = 4 MB per feature tile at the default 16384 columns)
-// mostly stay in L2.  If the
-// caller's list is row-sorted, as a COO list derived from CSR is, consecutive
-// edges of a block still share their Dst row, which L1 serves.
+// mostly stay in L2, and consecutive edges of a block share their Dst row, which L1
+// serves.
 //
 // Long feature rows are processed in tiles of 64 floats, one launch per tile:
 // tile t adds its 64-term partial dot product to Out[e] (the reference's x86
@@ -29,10 +29,15 @@ namespace {
 
 constexpr int kTile = 64;  // floats per tile: 16 lanes x float4 per edge
 
-__global__ void block_keys_kernel(const int32_t *col, int64_t nnz, int32_t block_cols, uint32_t *keys, int32_t *ids) {
+// Sort key of an edge: its column block and, below it when row_bits > 0, its row id, so that inside a block the
+// edges of one destination row sit together whatever order the caller listed them in.
+__global__ void block_keys_kernel(const int32_t *row, const int32_t *col, int64_t nnz, int32_t block_cols,
+                                  int32_t n_rows, int row_bits, uint32_t *keys, int32_t *ids) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
-    keys[i] = static_cast<uint32_t>(max(col[i], 0)) / static_cast<uint32_t>(block_cols);
+    uint32_t key = static_cast<uint32_t>(max(col[i], 0)) / static_cast<uint32_t>(block_cols);
+    if (row_bits > 0) key = (key << row_bits) | static_cast<uint32_t>(min(max(row[i], 0), n_rows - 1));
+    keys[i] = key;
     ids[i] = static_cast<int32_t>(i);
   }
 }
@@ -73,6 +78,12 @@ int sddmm_blocks_build(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_
     return FG_OK;
   int bits = 1;
   while ((int64_t{1} << bits) < n_blocks) ++bits;
+  // with room in a 32-bit key, order the edges of a block by destination row as well: consecutive edges then
+  // share their Dst row (served by L1) also when the caller's list was in no particular order
+  int row_bits = 1;
+  while ((int64_t{1} << row_bits) < n_rows) ++row_bits;
+  if (bits + row_bits > 32) row_bits = 0;
+  bits += row_bits;
 
   uint32_t *keys = nullptr, *keys_sorted = nullptr;
   int32_t *ids = nullptr;
@@ -87,14 +98,15 @@ int sddmm_blocks_build(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_
   if (err == hipSuccess) err = hipMalloc(&out->col_p, n * sizeof(int32_t));
   if (err == hipSuccess) {
     const int grid = static_cast<int>(std::min<int64_t>((nnz + 255) / 256, 65536));
-    block_keys_kernel<<<dim3(grid), dim3(256)>>>(col, nnz, static_cast<int32_t>(block_cols), keys, ids);
+    block_keys_kernel<<<dim3(grid), dim3(256)>>>(row, col, nnz, static_cast<int32_t>(block_cols),
+                                                 static_cast<int32_t>(n_rows), row_bits, keys, ids);
     err = hipGetLastError();
   }
   if (err == hipSuccess)
     err = hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, keys, keys_sorted, ids, out->pos_p,
                                              static_cast<int>(nnz), 0, bits, nullptr);
   if (err == hipSuccess) err = hipMalloc(&tmp, tmp_bytes ? tmp_bytes : 1);
-  if (err == hipSuccess)  // LSD radix sort: stable, so every block keeps the caller's edge order
+  if (err == hipSuccess)  // LSD radix sort: stable, so edges with equal keys keep the caller's order
     err = hipcub::DeviceRadixSort::SortPairs(tmp, tmp_bytes, keys, keys_sorted, ids, out->pos_p,
                                              static_cast<int>(nnz), 0, bits, nullptr);
   if (err == hipSuccess) {

@@ -186,9 +186,9 @@ FG_API int fg_sddmm_coo_general_f32(int64_t nnz, const int32_t *row, const int32
  * and whose column ids ascend inside every row (COO derived from CSR) it
  * rebuilds the row pointer and stores where every block of 16384 columns
  * starts inside every row ((n_cols/16384 + 3) * n_rows int32); for any other
- * list it stores the edge list re-ordered by blocks of 16384 columns (stable,
- * so each block keeps the caller's order) together with every edge's original
- * position: 12 bytes per edge, one device radix sort.  Results are always written in the
+ * list it stores the edge list re-ordered by blocks of 16384 columns and, inside
+ * a block, by destination row (stable otherwise) together with every edge's
+ * original position: 12 bytes per edge, one device radix sort.  Results are always written in the
  * caller's edge order; there is no edge_mapping to apply.  The plan BORROWS row
  * and col, which must stay alive and unchanged until fg_sddmm_plan_destroy.
  */
