@@ -25,7 +25,7 @@ struct Config {
   int spmm_vec = 0, spmm_lpr = 0, spmm_unroll = 0, spmm_scalar_path = -1, spmm_sorted = -1;
   int spmm_blocked = -1, spmm_block_cols = 0, spmm_pipeline = -1, spmm_pipe_blocks = 0;
   int spmm_buffer_loads = -1;
-  int spmm_multi = -1, spmm_multi_blocks = 0, spmm_multi_long = 0;
+  int spmm_multi = -1, spmm_multi_blocks = 0, spmm_multi_long = 0, spmm_tile_interleave = 0;
   int sddmm_group = 0, sddmm_batches = 0, sddmm_blocked = -1, sddmm_block_cols = 0;
   int sddmm_fast = -1, sddmm_buffer_loads = -1, sddmm_rows = -1, sddmm_rows_blocks = 0;
 };
@@ -63,6 +63,7 @@ struct SpmmArgs {
   const int4 *runs = nullptr;
   int32_t long_runs = 0;    // the first long_runs records are long runs: one wave each, in the first
   int32_t long_blocks = 0;  // long_blocks workgroups of the grid
+  int32_t interleave_tiles = 1;  // this many tiles alternate workgroup by workgroup along grid.x; the rest along grid.y
 };
 
 struct SpmmShape {

@@ -116,7 +116,7 @@ constexpr int kLongRounds = 8;  // rounds per batch of the long-run path; two ba
 
 template <int G, bool BUF, bool U24>
 __device__ __forceinline__ void spmm_long_runs(const SpmmArgs &a, const FeatRows<BUF, U24> &feat, int wave, int n_waves,
-                                               int lane, uint32_t lane_bytes, float *lds) {
+                                               int lane, uint32_t lane_bytes, float *lds, int tile) {
   constexpr int NG = kWaveSize / G;   // nonzeros per round
   constexpr int TW = 4 * G;           // floats per tile
   constexpr int R = kLongRounds;
@@ -125,7 +125,7 @@ __device__ __forceinline__ void spmm_long_runs(const SpmmArgs &a, const FeatRows
   const int g = lane / G;
   const int64_t F = a.F;
   const bool carry = a.accumulate != 0;
-  const int f1 = (a.tile_base + static_cast<int>(blockIdx.y)) * TW + lane;  // the float this lane sums
+  const int f1 = (a.tile_base + tile) * TW + lane;  // the float this lane sums
   const bool owner = lane < TW && f1 < a.F;
 
   auto load_ids = [&](int e, int rem, Ids &d) {
@@ -220,24 +220,30 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_multi_kernel(const SpmmArg
   const int gl = lane & (G - 1);
   const int g = lane / G;
   const bool hi_half = (lane & 8) != 0;
-  const int f0 = (a.tile_base + static_cast<int>(blockIdx.y)) * TW + gl * 4;
+  // `il` tiles alternate workgroup by workgroup along x, the rest of the tiles lie along y: workgroups go to the
+  // XCDs round-robin, so with il = 2 half of the XCDs work on each tile of a pair
+  const int il = max(a.interleave_tiles, 1);
+  const int tile = static_cast<int>(blockIdx.y) * il + static_cast<int>(blockIdx.x % il);
+  const int bx = static_cast<int>(blockIdx.x / il);
+  const int gx = static_cast<int>(gridDim.x / il);
+  const int f0 = (a.tile_base + tile) * TW + gl * 4;
   const bool fok = f0 < a.F;  // F is a multiple of 4: a lane's four floats exist together
   const int64_t F = a.F;
   const uint32_t lane_bytes = static_cast<uint32_t>(fok ? f0 : a.F - 4) * 4u;
   const FeatRows<BUF, U24> feat(a.feat, a.n_cols, F);
   const bool carry = a.accumulate != 0;
   // the first workgroups take the long runs (the records come by descending length), one wave per run
-  if (static_cast<int>(blockIdx.x) < a.long_blocks) {
+  if (bx < a.long_blocks) {
     __shared__ float products[kWavesPerBlock][kLongRounds * 256];  // per wave: a batch of rounds x 64 lanes x float4
-    spmm_long_runs<G>(a, feat, static_cast<int>(blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)),
-                      a.long_blocks * kWavesPerBlock, lane, lane_bytes, products[threadIdx.x >> 6]);
+    spmm_long_runs<G>(a, feat, static_cast<int>(bx * kWavesPerBlock + (threadIdx.x >> 6)),
+                      a.long_blocks * kWavesPerBlock, lane, lane_bytes, products[threadIdx.x >> 6], tile);
     return;
   }
-  const int n_waves = (gridDim.x - a.long_blocks) * kWavesPerBlock;
+  const int n_waves = (gx - a.long_blocks) * kWavesPerBlock;
   const int n = a.n_rows;
   const int n_items = (n - a.long_runs + NG - 1) / NG;
   int item = __builtin_amdgcn_readfirstlane(
-      static_cast<int>((blockIdx.x - a.long_blocks) * kWavesPerBlock + (threadIdx.x >> 6)));
+      static_cast<int>((bx - a.long_blocks) * kWavesPerBlock + (threadIdx.x >> 6)));
 
   auto bounds = [&](int it, int &lo, int &hi, int &row) {
     lo = hi = 0;
@@ -357,7 +363,9 @@ int launch_multi(const SpmmArgs &a, int64_t blocks, bool buf, bool u24, hipStrea
   constexpr int NG = kWaveSize / G;
   const int64_t n_items = (static_cast<int64_t>(a.n_rows) - a.long_runs + NG - 1) / NG;
   blocks = std::max<int64_t>(1, std::min<int64_t>(blocks, (n_items + kWavesPerBlock - 1) / kWavesPerBlock));
-  const dim3 grid(static_cast<unsigned>(blocks + a.long_blocks), static_cast<unsigned>(a.n_tiles));
+  const int il = std::max(a.interleave_tiles, 1);
+  if (a.n_tiles % il != 0) return fail(FG_EINVAL, "tile interleave %d does not divide %d tiles", il, a.n_tiles);
+  const dim3 grid(static_cast<unsigned>((blocks + a.long_blocks) * il), static_cast<unsigned>(a.n_tiles / il));
   if (buf && u24)
     spmm_multi_kernel<G, true, true><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
   else if (buf)

@@ -306,7 +306,8 @@ FG_API int64_t fg_probe_gather_rows_count(int32_t row_floats, int64_t n_gathers)
  * it applies; by default it runs unless one of the shape keys above is set;
  * read at plan creation and at launch), "spmm.multi_blocks" (its grid size),
  * "spmm.multi_long" (run length from which a run gets a wave of its own,
- * default 512; read at plan creation),
+ * default 512; read at plan creation), "spmm.tile_interleave" (feature tiles
+ * whose workgroups alternate inside one launch of that kernel: 1 or 2, default 2),
  * "sddmm.blocked" (0/1: never / always build and use column blocks, read at
  * plan creation), "sddmm.block_cols" (columns per block, read at plan creation),
  * "sddmm.group" (lanes per dot product: 1..16),

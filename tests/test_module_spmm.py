@@ -36,7 +36,7 @@ def _oracle(adj, feat_np, P=1):
 def config_guard():
     yield
     for key in ("spmm.vec", "spmm.lpr", "spmm.unroll", "spmm.block_cols", "spmm.pipe_blocks",
-                "spmm.multi_blocks", "spmm.multi_long"):
+                "spmm.multi_blocks", "spmm.multi_long", "spmm.tile_interleave"):
         _lib.config_set(key, 0)
     for key in ("spmm.scalar_path", "spmm.sorted", "spmm.blocked", "spmm.pipeline",
                 "spmm.buffer_loads", "spmm.multi"):
@@ -562,3 +562,22 @@ def test_launch_time_keys_may_change_after_the_plan_exists(config_guard):
         module.out_tvm.tensor.fill_(2.0)
         assert np.array_equal(module.run([x]).asnumpy(), want), (key, value)
     assert len(seen) >= 4                                  # the description, hence the launch, did change
+
+
+@pytest.mark.parametrize("interleave", [1, 2])
+@pytest.mark.parametrize("F", [128, 192, 256, 260])
+def test_tiles_of_one_launch_in_turn_or_one_after_the_other(config_guard, interleave, F):
+    """Column-block passes cover every feature tile in one launch; pairs of tiles may alternate workgroup by
+    workgroup (even tile counts) or tiles follow one another.  Same bits either way, partial last tile included."""
+    _lib.config_set("spmm.blocked", 1)
+    _lib.config_set("spmm.block_cols", 700)
+    _lib.config_set("spmm.tile_interleave", interleave)
+    adj = datasets.config_graph("c2-mini")
+    feat = datasets.spmm_operands(adj, F)
+    module = VanillaSpMMhip(adj)
+    text = module.lower_to_ir([placeholder(feat.shape)], {}, {})
+    n_tiles = (F + 63) // 64
+    assert "rows-per-wave" in text and "%d in turn" % (interleave if n_tiles % interleave == 0 else 1) in text
+    module.build([placeholder(feat.shape)], {}, {})
+    module.out_tvm.tensor.fill_(4.0)
+    assert np.array_equal(module.run([nd.array(feat, module.ctx)]).asnumpy(), _oracle(adj, feat))
