@@ -251,7 +251,7 @@ const fg::MultiRuns *multi_table(const fg_spmm_plan *plan, const fg::SpmmArgs &a
   const fg::Config &c = fg::config();
   if (c.spmm_multi == 0 || !fg::spmm_multi_applies(a) || !plan->multi_whole.rec) return nullptr;
   if (c.spmm_multi < 0 && !(feat_tiles == 0 && c.spmm_vec == 0 && c.spmm_lpr == 0 && c.spmm_unroll == 0 &&
-                            c.spmm_pipeline < 0 && c.spmm_scalar_path < 0 && c.spmm_sorted != 0))
+                            c.spmm_pipeline < 0 && c.spmm_sorted != 0))
     return nullptr;
   const int tile = fg::spmm_multi_tile(a.F);
   const fg::MultiRuns *blocked = &plan->multi_tile[multi_tile_index(tile)];
@@ -399,7 +399,6 @@ int *config_slot(const char *key) {
   if (!strcmp(key, "spmm.vec")) return &c.spmm_vec;
   if (!strcmp(key, "spmm.lpr")) return &c.spmm_lpr;
   if (!strcmp(key, "spmm.unroll")) return &c.spmm_unroll;
-  if (!strcmp(key, "spmm.scalar_path")) return &c.spmm_scalar_path;
   if (!strcmp(key, "spmm.sorted")) return &c.spmm_sorted;
   if (!strcmp(key, "spmm.blocked")) return &c.spmm_blocked;
   if (!strcmp(key, "spmm.block_cols")) return &c.spmm_block_cols;
@@ -850,7 +849,7 @@ int fg_check_indices(int64_t n, const int32_t *idx, int64_t bound, int64_t *n_ba
 int fg_config_set(const char *key, int32_t value) {
   int *slot = config_slot(key);
   if (!slot) return fg::fail(FG_EINVAL, "unknown configuration key '%s'", key ? key : "(null)");
-  const bool flag = slot == &fg::config().spmm_scalar_path || slot == &fg::config().spmm_sorted ||
+  const bool flag = slot == &fg::config().spmm_sorted ||
                     slot == &fg::config().spmm_blocked || slot == &fg::config().spmm_pipeline ||
                     slot == &fg::config().sddmm_blocked ||
                     slot == &fg::config().spmm_buffer_loads || slot == &fg::config().sddmm_fast ||
@@ -908,7 +907,7 @@ int fg_spmm_describe(const fg_spmm_plan *plan, int32_t H, int32_t D, int32_t fea
            "lanes/row-slot=%d tile=%d floats x %d tiles gathers-in-flight=%d rows=%s | %s, grid=%lld blocks x %d "
            "threads each",
            (long long)plan->n_rows, (long long)plan->n_cols, (long long)plan->nnz, plan->max_degree, H, D,
-           s.pipeline ? "wave-per-row(pipelined)" : (s.scalar_path ? "wave-per-row(scalar ids)" : "row-slot"), s.vec, s.lpr, s.tile_width(), a.n_tiles,
+           s.pipeline ? "wave-per-row(pipelined)" : "row-slot", s.vec, s.lpr, s.tile_width(), a.n_tiles,
            s.unroll, a.row_order ? "by-descending-degree" : "natural", passes,
            (long long)((waves + fg::kWavesPerBlock - 1) / fg::kWavesPerBlock), fg::kBlockThreads);
   return FG_OK;

@@ -22,7 +22,7 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 
 // Launch-shape overrides (0 = library default).
 struct Config {
-  int spmm_vec = 0, spmm_lpr = 0, spmm_unroll = 0, spmm_scalar_path = -1, spmm_sorted = -1;
+  int spmm_vec = 0, spmm_lpr = 0, spmm_unroll = 0, spmm_sorted = -1;
   int spmm_blocked = -1, spmm_block_cols = 0, spmm_pipeline = -1, spmm_pipe_blocks = 0;
   int spmm_buffer_loads = -1;
   int spmm_multi = -1, spmm_multi_blocks = 0, spmm_multi_long = 0, spmm_tile_interleave = 0;
@@ -67,7 +67,7 @@ struct SpmmArgs {
 };
 
 struct SpmmShape {
-  int vec, lpr, unroll, scalar_path;
+  int vec, lpr, unroll;
   int pipeline = 0;       // wave-per-row kernel that keeps three rows in flight
   int pipe_blocks = 0;    // its grid size (workgroups per feature tile)
   int tile_width() const { return vec * lpr; }

@@ -152,80 +152,6 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_slot_kernel(const SpmmArgs
   if (fok) *reinterpret_cast<V *>(op) = acc;
 }
 
-// Wave-per-(row, tile) kernel (LPR = 64): the row bounds and each neighbour's
-// column id and value live in scalar registers, so a gather is one vector load
-// from a scalar base plus the lane's fixed offset, with no per-lane address
-// arithmetic.
-template <int VEC, int U, bool MH>
-__global__ __launch_bounds__(kBlockThreads) void spmm_wave_kernel(const SpmmArgs a) {
-  using V = typename VecOf<VEC>::type;
-  constexpr int TW = VEC * kWaveSize;
-  const int lane = threadIdx.x & (kWaveSize - 1);
-  const int64_t slot = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
-  if (slot >= a.n_slots) return;
-  const int tile = __builtin_amdgcn_readfirstlane(static_cast<int>(slot / a.n_rows));
-  const int i = __builtin_amdgcn_readfirstlane(static_cast<int>(slot - static_cast<int64_t>(tile) * a.n_rows));
-  const int row = __builtin_amdgcn_readfirstlane(a.row_order ? a.row_order[i] : i);
-  const int f0 = (a.tile_base + tile) * TW + lane * VEC;
-  const bool fok = f0 < a.F;
-  const int head = (MH && fok) ? f0 / a.D : 0;
-  const int64_t F = a.F;
-  const float *fp = a.feat + (fok ? f0 : a.F - VEC);  // lanes past a partial tile re-read its last group and never store
-  const float *wp = a.w + head;
-  int e = __builtin_amdgcn_readfirstlane(a.seg_lo ? a.seg_lo[i] : a.indptr[row]);
-  const int end = __builtin_amdgcn_readfirstlane(a.seg_lo ? a.seg_hi[i] : a.indptr[row + 1]);
-  V acc = vzero<VEC>();
-  float *const op = a.out + static_cast<int64_t>(row) * F + f0;
-  if (a.accumulate) {
-    if (e >= end) return;  // nothing of this row in this column block: the carried sum stays as it is
-    if (fok) acc = *reinterpret_cast<const V *>(op);
-  }
-  for (; e < end; e += kWaveSize) {
-    const int n = min(kWaveSize, end - e);
-    int my_col = 0;
-    float my_val = 0.0f;
-    if (lane < n) {
-      my_col = a.indices[e + lane];
-      if (!MH) my_val = a.w[e + lane];
-    }
-    int j = 0;
-    for (; j + U <= n; j += U) {
-      V x[U];
-      float v[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int c = __builtin_amdgcn_readlane(my_col, j + u);
-        x[u] = *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F);
-        if (MH)
-          v[u] = wp[static_cast<int64_t>(e + j + u) * a.H];
-        else
-          v[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_val), j + u));
-      }
-#pragma unroll
-      for (int u = 0; u < U; ++u) axpy(acc, v[u], x[u]);
-    }
-    if (j < n) {  // fewer than U left: one masked batch, so these gathers overlap too
-      V x[U];
-      float v[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const bool live = j + u < n;  // wave-uniform
-        const int c = __builtin_amdgcn_readlane(my_col, (j + u) & (kWaveSize - 1));
-        x[u] = live ? *reinterpret_cast<const V *>(fp + static_cast<int64_t>(c) * F) : vzero<VEC>();
-        if (MH)
-          v[u] = live ? wp[static_cast<int64_t>(e + j + u) * a.H] : 0.0f;
-        else
-          v[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_val), (j + u) & (kWaveSize - 1)));
-      }
-#pragma unroll
-      for (int u = 0; u < U; ++u)
-        if (j + u < n) axpy(acc, v[u], x[u]);
-    }
-  }
-  if (fok) *reinterpret_cast<V *>(op) = acc;
-}
-
-
 // One neighbour row's VEC floats for this lane.  With BUF the feature matrix is
 // addressed as a buffer resource: the load takes the lane's fixed byte offset in
 // a vector register and the row's byte offset (column id * row bytes) in a
@@ -430,18 +356,6 @@ int launch_slot(const SpmmArgs &a, hipStream_t stream) {
 }
 
 template <int VEC, int U>
-int launch_wave(const SpmmArgs &a, hipStream_t stream) {
-  const int64_t blocks = (a.n_slots + kWavesPerBlock - 1) / kWavesPerBlock;
-  if (blocks > 0x7fffffffLL) return fail(FG_EUNSUPPORTED, "SpMM launch needs %lld blocks", (long long)blocks);
-  if (a.H > 1)
-    spmm_wave_kernel<VEC, U, true><<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(a);
-  else
-    spmm_wave_kernel<VEC, U, false><<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(a);
-  FG_HIP_TRY(hipGetLastError());
-  return FG_OK;
-}
-
-template <int VEC, int U>
 int launch_pipe(const SpmmArgs &a, const SpmmShape &s, hipStream_t stream) {
   if (!a.seg_lo || !a.row_order) return fail(FG_EINVAL, "the pipelined kernel needs the plan's row list and bounds");
   // a fixed number of resident waves, each walking many rows
@@ -475,13 +389,6 @@ int dispatch_unroll(const SpmmArgs &a, const SpmmShape &s, hipStream_t stream) {
       case 8: return launch_pipe<VEC, 8>(a, s, stream);
       case 16: return launch_pipe<VEC, 16>(a, s, stream);
       case 32: return launch_pipe<VEC, 32>(a, s, stream);
-    }
-  } else if (LPR == kWaveSize && s.scalar_path) {
-    switch (s.unroll) {
-      case 4: return launch_wave<VEC, 4>(a, stream);
-      case 8: return launch_wave<VEC, 8>(a, stream);
-      case 16: return launch_wave<VEC, 16>(a, stream);
-      case 32: return launch_wave<VEC, 32>(a, stream);
     }
   } else {
     switch (s.unroll) {
@@ -547,8 +454,6 @@ SpmmShape spmm_choose_shape(const SpmmArgs &a, int feat_tiles) {
   if (lanes > kWaveSize) lanes = kWaveSize;
   s.lpr = cfg.spmm_lpr > 0 ? cfg.spmm_lpr : lanes;
   s.unroll = cfg.spmm_unroll > 0 ? cfg.spmm_unroll : (two_rows ? 4 : s.lpr == 32 ? 32 : (s.lpr >= 16 ? 16 : 8));
-  s.scalar_path = cfg.spmm_scalar_path >= 0 ? cfg.spmm_scalar_path : 1;
-  if (s.lpr != kWaveSize) s.scalar_path = 0;
   s.pipeline = cfg.spmm_pipeline >= 0 ? cfg.spmm_pipeline : 1;
   if (s.lpr != kWaveSize || !a.seg_lo || !a.row_order) s.pipeline = 0;
   s.pipe_blocks = cfg.spmm_pipe_blocks > 0 ? cfg.spmm_pipe_blocks : 16384;

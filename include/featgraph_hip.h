@@ -294,8 +294,7 @@ FG_API int64_t fg_probe_gather_rows_count(int32_t row_floats, int64_t n_gathers)
  * the kernel choice changes.
  * Keys: "spmm.vec" (floats per lane: 1, 2, 4), "spmm.lpr" (lanes per row
  * slot: 8, 16, 32, 64), "spmm.unroll" (gathers in flight per lane: 4, 8, 16),
- * "spmm.scalar_path" (0/1: wave-per-row variant that keeps column ids in
- * scalar registers), "spmm.sorted" (0/1: visit rows by descending degree or
+ * "spmm.sorted" (0/1: visit rows by descending degree or
  * in natural order), "spmm.blocked" (0/1: never / always run SpMM as one pass
  * per column block when the plan has blocks; read at plan creation and at
  * launch), "spmm.block_cols" (columns per block, read at plan creation),

@@ -65,15 +65,15 @@ def test_config_store_round_trip():
     try:
         _lib.config_set("spmm.vec", 2)
         assert _lib.config_get("spmm.vec") == 2
-        _lib.config_set("spmm.scalar_path", 1)
-        assert _lib.config_get("spmm.scalar_path") == 1
-        _lib.config_set("spmm.scalar_path", -1)
-        assert _lib.config_get("spmm.scalar_path") == -1
+        _lib.config_set("spmm.pipeline", 1)
+        assert _lib.config_get("spmm.pipeline") == 1
+        _lib.config_set("spmm.pipeline", -1)
+        assert _lib.config_get("spmm.pipeline") == -1
         with pytest.raises(_lib.FeatGraphError):
             _lib.config_set("no.such.key", 1)
     finally:
         _lib.config_set("spmm.vec", 0)
-        _lib.config_set("spmm.scalar_path", -1)
+        _lib.config_set("spmm.pipeline", -1)
 
 
 def test_sddmm_launch_description_is_host_only():

@@ -38,7 +38,7 @@ def config_guard():
     for key in ("spmm.vec", "spmm.lpr", "spmm.unroll", "spmm.block_cols", "spmm.pipe_blocks",
                 "spmm.multi_blocks", "spmm.multi_long", "spmm.tile_interleave"):
         _lib.config_set(key, 0)
-    for key in ("spmm.scalar_path", "spmm.sorted", "spmm.blocked", "spmm.pipeline",
+    for key in ("spmm.sorted", "spmm.blocked", "spmm.pipeline",
                 "spmm.buffer_loads", "spmm.multi"):
         _lib.config_set(key, -1)
 
@@ -110,31 +110,15 @@ def test_powerlaw_graph_with_hub_rows(F):
 
 
 @pytest.mark.parametrize("key,values", [("spmm.vec", [1, 2, 4]), ("spmm.lpr", [8, 16, 32, 64]),
-                                        ("spmm.unroll", [4, 8, 16]), ("spmm.scalar_path", [0, 1]),
-                                        ("spmm.sorted", [0, 1])])
+                                        ("spmm.unroll", [4, 8, 16]), ("spmm.sorted", [0, 1])])
 @pytest.mark.parametrize("F", [64, 200])
 def test_every_launch_shape_gives_the_same_bits(config_guard, key, values, F):
     adj = datasets.config_graph("c2-mini")
     feat = datasets.spmm_operands(adj, F)
     want = _oracle(adj, feat)
     for v in values:
-        if key == "spmm.scalar_path":
-            _lib.config_set("spmm.lpr", 64)
         _lib.config_set(key, v)
         assert np.array_equal(_run_spmm(adj, feat), want), "%s=%d" % (key, v)
-
-
-@pytest.mark.parametrize("vec", [1, 2, 4])
-@pytest.mark.parametrize("unroll", [4, 16])
-def test_scalar_path_variants(config_guard, vec, unroll):
-    adj = datasets.config_graph("c2-mini")
-    feat = datasets.spmm_operands(adj, 256)
-    _lib.config_set("spmm.lpr", 64)
-    _lib.config_set("spmm.scalar_path", 1)
-    _lib.config_set("spmm.pipeline", 0)
-    _lib.config_set("spmm.vec", vec)
-    _lib.config_set("spmm.unroll", unroll)
-    assert np.array_equal(_run_spmm(adj, feat), _oracle(adj, feat))
 
 
 @pytest.mark.parametrize("vec", [1, 2, 4])
@@ -384,15 +368,14 @@ def test_very_many_partitions_keep_the_bounds_table_only(config_guard):
 
 # ---------------------------------------------------------------- column-blocked passes
 @pytest.mark.parametrize("block_cols", [7, 100, 1500])
-@pytest.mark.parametrize("shape", [(4, 16, 0), (1, 64, 1), (1, 64, 0), (2, 32, 0), (1, 32, 0), (1, 64, 2), (2, 64, 2)])
+@pytest.mark.parametrize("shape", [(4, 16, 0), (1, 64, 0), (2, 32, 0), (1, 32, 0), (1, 64, 2), (2, 64, 2)])
 def test_column_blocked_passes_give_the_same_bits(config_guard, block_cols, shape):
     adj = datasets.config_graph("c2-mini")
     _lib.config_set("spmm.blocked", 1)
     _lib.config_set("spmm.block_cols", block_cols)
-    vec, lpr, kind = shape                      # kind: 0 row-slot kernel, 1 scalar-id kernel, 2 pipelined kernel
+    vec, lpr, kind = shape                      # kind: 0 row-slot kernel, 2 pipelined kernel
     _lib.config_set("spmm.vec", vec)
     _lib.config_set("spmm.lpr", lpr)
-    _lib.config_set("spmm.scalar_path", int(kind == 1))
     _lib.config_set("spmm.pipeline", int(kind == 2))
     for F in (64, 200):
         feat = datasets.spmm_operands(adj, F)
@@ -500,8 +483,8 @@ def test_multihead_spmm_with_one_head_is_the_vanilla_kernel(config_guard):
         assert np.array_equal(_run_mh(adj, feat, adj.data.reshape(-1, 1).copy())[:, 0], vanilla)
 
 
-@pytest.mark.parametrize("key,values", [("spmm.vec", [1, 2, 4]), ("spmm.lpr", [8, 32, 64]), ("spmm.scalar_path", [1]),
-                                        ("spmm.pipeline", [1])])
+@pytest.mark.parametrize("key,values", [("spmm.vec", [1, 2, 4]), ("spmm.lpr", [8, 32, 64]),
+                                        ("spmm.pipeline", [0, 1])])
 def test_multihead_launch_shapes_give_the_same_bits(config_guard, key, values):
     adj = datasets.config_graph("c4-mini")
     H, D = 8, 32
@@ -509,7 +492,7 @@ def test_multihead_launch_shapes_give_the_same_bits(config_guard, key, values):
     w = datasets.softmax_edge_weights(adj, H)
     want = ref.spmm_mh(adj.indptr, adj.indices, w, feat)
     for v in values:
-        if key in ("spmm.scalar_path", "spmm.pipeline"):
+        if key == "spmm.pipeline":
             _lib.config_set("spmm.lpr", 64)
         _lib.config_set(key, v)
         assert np.array_equal(_run_mh(adj, feat, w), want), "%s=%d" % (key, v)
