@@ -74,6 +74,12 @@ def mh_spmm_alg_bytes(nnz, n_rows, H, D):
     return nnz * (4 + 4 * H + 4 * H * D) + n_rows * (4 + 4 * H * D)
 
 
+def mh_attention_alg_bytes(nnz, n_rows, H, D, shared):
+    """Gather model of the fused attention operator: per nonzero the id and one (key = value) or two gathered rows,
+    per destination row its bounds, the query and the result."""
+    return nnz * (4 + (1 if shared else 2) * 4 * H * D) + n_rows * (8 + 8 * H * D)
+
+
 def committed_traffic(op, graph, F):
     """(bytes per launch across the L2 boundary, source file) from the counter summary in profiles/, or (None, None)."""
     rel = os.path.join("profiles", "%s_%s_counters.txt" % (op, graph))
@@ -116,7 +122,7 @@ def main():
     ap.add_argument("--feat-len", type=int, default=64, help="feature length of the timed step")
     ap.add_argument("--graph", default="c2", help="named synthetic configuration (featgraph_amd.datasets.CONFIGS)")
     ap.add_argument("--only", choices=["all", "spmm", "sddmm", "copy", "mh_sddmm", "mh_spmm", "mh_sddmm_softmax",
-                                       "gather_probe"],
+                                       "mh_attention", "mh_attention_kv", "gather_probe"],
                     default="all",
                     help="spmm / sddmm / copy / gather_probe: run just that kernel (for profiler runs), no sweep, no "
                          "CPU leg; mh_sddmm / mh_spmm: the multi-head operators (8 heads of --feat-len floats, use "
@@ -132,8 +138,8 @@ def main():
     import numpy as np
     import torch
     from featgraph_amd import _lib, datasets, nd, placeholder
-    from featgraph_amd.module import (EdgeSoftmaxhip, MultiHeadSDDMMhip, MultiHeadSDDMMSoftmaxhip, MultiHeadSpMMhip,
-                                      VanillaSDDMMhip, VanillaSpMMhip)
+    from featgraph_amd.module import (EdgeSoftmaxhip, MultiHeadAttentionhip, MultiHeadSDDMMhip,
+                                      MultiHeadSDDMMSoftmaxhip, MultiHeadSpMMhip, VanillaSDDMMhip, VanillaSpMMhip)
 
     L = _lib.lib()  # fail now if the HIP library is missing
     if not torch.cuda.is_available():
@@ -224,6 +230,16 @@ def main():
             op.build([placeholder((n_c, H, D)), placeholder((n_r, H, D))], {}, {})
             ins = [src, dst]
             b, b_min = mh_sddmm_alg_bytes(e, H, D), 8 * e + 4 * H * e + 4 * H * D * (n_r + n_c)
+        elif kind in ("mh_attention", "mh_attention_kv"):
+            # scores, softmax and weighted sum in one kernel; "mh_attention": the vertex features are key and value
+            shared = kind == "mh_attention"
+            op = MultiHeadAttentionhip(graph_adj)
+            src, dst = device_normal((n_c, H, D), 11 + D), device_normal((n_r, H, D), 12 + D)
+            src *= 0.25
+            ins = [src, dst] if shared else [src, dst, device_normal((n_c, H, D), 14 + D)]
+            op.build([placeholder(tuple(x.shape)) for x in ins], {}, {})
+            b = mh_attention_alg_bytes(e, n_r, H, D, shared)
+            b_min = 4 * e + 8 * n_r + 4 * H * D * (2 * n_r + (1 if shared else 2) * n_c)
         else:
             op = MultiHeadSpMMhip(graph_adj)
             src = device_normal((n_c, H, D), 13 + D)
@@ -269,12 +285,22 @@ def main():
                 want = ref.edge_softmax(graph_adj.indptr[:n_check + 1], scores)
                 ok = bool(np.all(np.abs(out[:m] - want) <= 1e-6 + 1e-4 * np.abs(want)))
                 row["parity"] = {"within_rtol1e-4_atol1e-6_of_cpu_checker": ok, "edges_checked": m}
+            elif kind in ("mh_attention", "mh_attention_kv"):
+                # the first rows (the three CPU checkers one after the other on their sub-matrix) against the kernel
+                n_check = int(np.searchsorted(graph_adj.indptr, 1_500_000))
+                m = int(graph_adj.indptr[n_check])
+                hosts = [x.cpu().numpy() for x in ins]
+                want = ref.attention_mh(graph_adj.indptr[:n_check + 1], graph_adj.indices[:m], hosts[0],
+                                        hosts[1][:n_check], hosts[2] if len(hosts) == 3 else None)
+                ok = bool(np.all(np.abs(out[:n_check] - want) <= 1e-5 + 1e-4 * np.abs(want)))
+                row["parity"] = {"within_rtol1e-4_atol1e-5_of_cpu_checker": ok, "rows_checked": n_check,
+                                 "edges_checked": m}
             else:
                 want = ref.spmm_mh(graph_adj.indptr, graph_adj.indices, w.cpu().numpy(), src.cpu().numpy())
                 row["parity"] = {"bit_exact_vs_cpu_checker": bool(np.array_equal(out, want))}
         return row
 
-    if args.only in ("mh_sddmm", "mh_spmm", "mh_sddmm_softmax"):
+    if args.only in ("mh_sddmm", "mh_spmm", "mh_sddmm_softmax", "mh_attention", "mh_attention_kv"):
         row = mh_case(args.only, adj, F, args.steps, args.warmup, False)
         row.update({"kernel": args.only, "graph": args.graph})
         print(json.dumps(row))
@@ -472,6 +498,18 @@ def main():
         torch.cuda.empty_cache()
         mh.append(mh_case("mh_spmm", big, 64, 5, 1, check))
         log("mh_spmm D=64: %.3f ms (%.2f of the HBM roofline by algorithmic bytes)" % (mh[-1]["ms"], mh[-1]["frac"]))
+        torch.cuda.empty_cache()
+        # the whole layer in one kernel: scores, softmax and weighted sum, with the vertex features as key and value
+        # (one gather per neighbour) and with a separate value matrix (two)
+        chain_ms = {r["D"]: r["ms"] for r in mh if r["op"] == "mh_sddmm_softmax"}
+        spmm_ms = mh[-1]["ms"]
+        for kind in ("mh_attention", "mh_attention_kv"):
+            mh.append(mh_case(kind, big, 64, 5, 1, check))
+            mh[-1]["chain_ms"] = chain_ms[64] + spmm_ms
+            mh[-1]["speedup_over_chain"] = mh[-1]["chain_ms"] / mh[-1]["ms"]
+            torch.cuda.empty_cache()
+            log("%s D=64: %.3f ms (scores + softmax, then multi-head SpMM: %.3f ms)" % (
+                kind, mh[-1]["ms"], mh[-1]["chain_ms"]))
         result["multi_head"] = {"graph": "c4: %d vertices, %d edges" % (big.shape[0], big.nnz), "rows": mh,
                                 "note": "1.25 - 5 GB of features and mean degree 25: nearly every neighbour gather "
                                         "goes to HBM.  `frac` is algorithmic bytes / time / 8 TB/s (above 1 for SDDMM "

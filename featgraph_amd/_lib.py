@@ -32,6 +32,7 @@ SIGNATURES = {
     "fg_sddmm_coo_plan_f32": (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _p]),
     "fg_edge_softmax_csr_f32": (ctypes.c_int, [_i64, _p, _p, _p, _i32, _p]),
     "fg_sddmm_softmax_plan_f32": (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _p]),
+    "fg_attention_csr_mh_f32": (ctypes.c_int, [_p, _p, _p, _p, _p, _i32, _i32, _p]),
     "fg_sddmm_plan_describe": (ctypes.c_int, [_p, _i32, _i32, ctypes.c_char_p, _i64]),
     "fg_check_indices": (ctypes.c_int, [_i64, _p, _i64, ctypes.POINTER(_i64), _p]),
     "fg_probe_gather_f32": (ctypes.c_int, [_p, _i64, _i32, _i32, _i32, _i64, _p, _p]),

@@ -417,6 +417,7 @@ int *config_slot(const char *key) {
   if (!strcmp(key, "sddmm.buffer_loads")) return &c.sddmm_buffer_loads;
   if (!strcmp(key, "sddmm.rows")) return &c.sddmm_rows;
   if (!strcmp(key, "sddmm.rows_blocks")) return &c.sddmm_rows_blocks;
+  if (!strcmp(key, "attention.blocks")) return &c.attention_blocks;
   return nullptr;
 }
 
@@ -794,6 +795,23 @@ int fg_sddmm_softmax_plan_f32(const fg_sddmm_plan *plan, const float *src, const
     return fg::sddmm_softmax_launch(plan->rows->row_order, plan->indptr, plan->col, src, dst, out, n, H, D, st);
   if (int rc = fg_sddmm_coo_plan_f32(plan, src, dst, out, H, D, stream)) return rc;
   return fg::edge_softmax_launch(plan->indptr, out, out, n, H, st);
+}
+
+int fg_attention_csr_mh_f32(const fg_spmm_plan *plan, const float *key, const float *query, const float *value,
+                            float *out, int32_t H, int32_t D, void *stream) {
+  if (!plan) return fg::fail(FG_EINVAL, "plan is null");
+  if (int rc = check_heads(H, D)) return rc;
+  if (plan->n_rows == 0) return FG_OK;
+  if (int rc = check_device(plan->device)) return rc;
+  if (!key || !query || !value || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
+  if (!fg::attention_fused_applies(key, query, value, out, H, D))
+    return fg::fail(FG_EUNSUPPORTED,
+                    "the fused attention kernel has no layout for H = %d, D = %d with these operand alignments: run "
+                    "fg_sddmm_softmax_plan_f32 and fg_spmm_csr_mh_f32 one after the other",
+                    H, D);
+  const int32_t n = static_cast<int32_t>(plan->n_rows);
+  return fg::attention_launch(plan->row_order, plan->seg, plan->seg + static_cast<int64_t>(plan->n_blocks) * n,
+                              plan->indices, key, query, value, out, n, H, D, static_cast<hipStream_t>(stream));
 }
 
 int fg_sddmm_plan_describe(const fg_sddmm_plan *plan, int32_t H, int32_t D, char *buf, int64_t cap) {

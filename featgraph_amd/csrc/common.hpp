@@ -28,6 +28,7 @@ struct Config {
   int spmm_multi = -1, spmm_multi_blocks = 0, spmm_multi_long = 0, spmm_tile_interleave = 0;
   int sddmm_group = 0, sddmm_batches = 0, sddmm_blocked = -1, sddmm_block_cols = 0;
   int sddmm_fast = -1, sddmm_buffer_loads = -1, sddmm_rows = -1, sddmm_rows_blocks = 0;
+  int attention_blocks = 0;
 };
 Config &config();
 
@@ -159,6 +160,13 @@ int edge_softmax_launch(const int32_t *indptr, const float *scores, float *out, 
 bool sddmm_softmax_fused_applies(const float *src, const float *dst, int32_t H, int32_t D);
 int sddmm_softmax_launch(const int32_t *row_order, const int32_t *indptr, const int32_t *indices, const float *src,
                          const float *dst, float *out, int32_t n_rows, int32_t H, int32_t D, hipStream_t stream);
+
+// Multi-head SDDMM, edge softmax and multi-head SpMM as one kernel (attention.hip).
+bool attention_fused_applies(const float *key, const float *query, const float *value, const float *out, int32_t H,
+                             int32_t D);
+int attention_launch(const int32_t *row_order, const int32_t *seg_lo, const int32_t *seg_hi, const int32_t *indices,
+                     const float *key, const float *query, const float *value, float *out, int32_t n_rows, int32_t H,
+                     int32_t D, hipStream_t stream);
 
 inline bool aligned_to(const void *p, uintptr_t bytes) { return (reinterpret_cast<uintptr_t>(p) & (bytes - 1)) == 0; }
 

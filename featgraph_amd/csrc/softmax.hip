@@ -22,25 +22,10 @@
 #include <cmath>
 
 #include "common.hpp"
+#include "rowlayout.hpp"
 
 namespace fg {
 namespace {
-
-template <int CTRL>
-__device__ __forceinline__ float dpp_add(float x) {
-  const int y = __builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, false);
-  return x + __int_as_float(y);
-}
-
-// Sum over aligned groups of G lanes (G <= 16); every lane of the group gets the total.
-template <int G>
-__device__ __forceinline__ float group_sum(float x) {
-  if (G >= 2) x = dpp_add<0xB1>(x);   // quad_perm [1,0,3,2]
-  if (G >= 4) x = dpp_add<0x4E>(x);   // quad_perm [2,3,0,1]
-  if (G >= 8) x = dpp_add<0x141>(x);  // row_half_mirror
-  if (G >= 16) x = dpp_add<0x140>(x); // row_mirror
-  return x;
-}
 
 // Running softmax state: m = largest score seen, l = sum of exp(score - m).
 struct MaxSum {
@@ -126,26 +111,6 @@ struct FusedArgs {
   float *out;        // [nnz, H]
   int32_t n_rows;
 };
-
-template <int VW>
-struct Floats {
-  float v[VW];
-};
-
-template <int VW>
-__device__ __forceinline__ Floats<VW> load_floats(const float *p) {
-  Floats<VW> r;
-  if constexpr (VW == 1) {
-    r.v[0] = *p;
-  } else if constexpr (VW == 2) {
-    const float2 q = *reinterpret_cast<const float2 *>(p);
-    r.v[0] = q.x, r.v[1] = q.y;
-  } else {
-    const float4 q = *reinterpret_cast<const float4 *>(p);
-    r.v[0] = q.x, r.v[1] = q.y, r.v[2] = q.z, r.v[3] = q.w;
-  }
-  return r;
-}
 
 // Layout of a vertex row (H * D floats) over a wave: NV chunks of 64 * VW floats; in chunk k lane l holds the
 // VW floats at k * 64 * VW + l * VW, so every load instruction of a gather covers consecutive addresses.  LC =
@@ -268,23 +233,6 @@ int launch_fused(const FusedArgs &a, hipStream_t stream) {
   return FG_OK;
 }
 
-// The layout for (H, D), or false when the fused kernel has none: the widest load for which a head spans 4, 8
-// or 16 lanes of a chunk and the row is one or two chunks.
-bool fused_layout(int32_t H, int32_t D, int *lc, int *vw, int *nv) {
-  for (int w = 4; w >= 1; w >>= 1) {
-    if (D % w != 0) continue;
-    const int c = D / w;
-    if (c != 4 && c != 8 && c != 16) continue;
-    const int hc = kWaveSize / c;
-    if (H % hc != 0) continue;
-    const int n = H / hc;
-    if ((n != 1 && n != 2) || c % n != 0) continue;
-    *lc = c, *vw = w, *nv = n;
-    return true;
-  }
-  return false;
-}
-
 }  // namespace
 
 int edge_softmax_launch(const int32_t *indptr, const float *scores, float *out, int32_t n_rows, int32_t H,
@@ -303,7 +251,7 @@ int edge_softmax_launch(const int32_t *indptr, const float *scores, float *out, 
 // Whether the fused kernel covers this shape (see fused_layout) with operands aligned for its loads.
 bool sddmm_softmax_fused_applies(const float *src, const float *dst, int32_t H, int32_t D) {
   int lc, vw, nv;
-  if (H < 1 || D < 1 || !fused_layout(H, D, &lc, &vw, &nv)) return false;
+  if (H < 1 || D < 1 || !row_layout(H, D, &lc, &vw, &nv)) return false;
   return aligned_to(src, vw * 4) && aligned_to(dst, vw * 4);
 }
 
@@ -319,7 +267,7 @@ int sddmm_softmax_launch(const int32_t *row_order, const int32_t *indptr, const 
   a.out = out;
   a.n_rows = n_rows;
   int lc, vw, nv;
-  if (!fused_layout(H, D, &lc, &vw, &nv))
+  if (!row_layout(H, D, &lc, &vw, &nv))
     return fail(FG_EUNSUPPORTED, "the fused score + softmax kernel does not cover H = %d, D = %d", H, D);
 #define FG_FUSED_CASE(LC, VW, NV) \
   if (lc == LC && vw == VW && nv == NV) return launch_fused<LC, VW, NV>(a, stream);

@@ -2,3 +2,4 @@ from .sddmm import VanillaSDDMMhip, MultiHeadSDDMMhip
 from .spmm import VanillaSpMMhip, MultiHeadSpMMhip
 from .general import GeneralizedSpMMhip, GeneralizedSDDMMhip, VanillaSpMMGradhip
 from .softmax import EdgeSoftmaxhip, MultiHeadSDDMMSoftmaxhip
+from .attention import MultiHeadAttentionhip

@@ -241,6 +241,25 @@ FG_API int fg_edge_softmax_csr_f32(int64_t n_rows, const int32_t *indptr, const 
 FG_API int fg_sddmm_softmax_plan_f32(const fg_sddmm_plan *plan, const float *src, const float *dst, float *out,
                                      int32_t H, int32_t D, void *stream);
 
+/* Multi-head SDDMM, edge softmax and multi-head SpMM as one operator (no
+ * counterpart in the reference, which has the two ends as separate operators:
+ * the multi-head scores of op/vanilla_sddmm.py:35-47 and the multi-head SpMM
+ * of its benchmarks):
+ *   out[r, h, :] = sum over the nonzeros e of row r of A[e, h] * value[indices[e], h, :],
+ *   A[e, h] = softmax over the row's nonzeros of sum_d key[indices[e], h, d] * query[r, h, d].
+ * key, value [n_cols, H, D]; query, out [n_rows, H, D]; rows without nonzeros
+ * give zeros.  The scores and weights never exist in memory; when value == key
+ * every neighbour row is gathered once for both uses.  Float32 throughout with a
+ * running (max, sum) softmax: agrees with the three operators run one after the
+ * other within rtol 1e-4 / atol 1e-5, not bit for bit (the weighted sum is
+ * rescaled whenever the running maximum grows).  Shapes: those of the fused
+ * score + softmax kernel (a head spans 4, 8 or 16 lanes of 1, 2 or 4 floats, a
+ * vertex row is 64 or 128 such loads: H = 8 with D in {8, ..., 64}, H = 4 with
+ * D in {16, 32, 64}, ...); FG_EUNSUPPORTED otherwise, and the caller runs
+ * fg_sddmm_softmax_plan_f32 and fg_spmm_csr_mh_f32 instead. */
+FG_API int fg_attention_csr_mh_f32(const fg_spmm_plan *plan, const float *key, const float *query, const float *value,
+                                   float *out, int32_t H, int32_t D, void *stream);
+
 /*
  * Multi-head SDDMM (no counterpart in the reference; the edge function of
  * op/vanilla_sddmm.py:47 per head): Out[e, h] = sum_d src[col[e], h, d] * dst[row[e], h, d].
@@ -313,7 +332,8 @@ FG_API int64_t fg_probe_gather_rows_count(int32_t row_floats, int64_t n_gathers)
  * "sddmm.batches" (64-edge batches per wave), "sddmm.fast" (0/1: unrolled
  * kernel for D in 16..512), "sddmm.buffer_loads" (0/1), "sddmm.rows" (0/1:
  * never / always use the row-run kernel when the plan has a row plan; read at
- * plan creation and at launch), "sddmm.rows_blocks" (its grid size).  Value 0 restores the default of
+ * plan creation and at launch), "sddmm.rows_blocks" (its grid size),
+ * "attention.blocks" (grid size of the fused attention kernel).  Value 0 restores the default of
  * a size; for the 0/1 flags a negative value does.
  * The spmm.* keys change the launch shape only; "sddmm.group" also changes the
  * shape of the summation tree, i.e. the last bits of an SDDMM result.

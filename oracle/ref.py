@@ -192,3 +192,15 @@ def edge_softmax(indptr, scores):
     _check(lib().fgref_edge_softmax(_i64(n_dst), _i64(H), _ptr(indptr), _ptr(scores), _ptr(out)),
            "fgref_edge_softmax")
     return out
+
+
+def attention_mh(indptr, indices, key, query, value=None):
+    """out[r, h, :] = sum over row r's nonzeros e of softmax_e(key[indices[e], h] . query[r, h]) * value[indices[e], h, :].
+
+    The three checkers above one after the other: sddmm_mh (scores, float32), edge_softmax (binary64 inside),
+    spmm_mh (sequential float32 sum).  value defaults to key.  Rows without nonzeros give zeros.
+    """
+    indptr, indices = _arr(indptr, np.int32), _arr(indices, np.int32)
+    row = np.repeat(np.arange(indptr.shape[0] - 1, dtype=np.int32), np.diff(indptr))
+    weights = edge_softmax(indptr, sddmm_mh(row, indices, key, query))
+    return spmm_mh(indptr, indices, weights, key if value is None else value)

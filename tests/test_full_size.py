@@ -237,6 +237,39 @@ def test_c4_fused_scores_and_softmax(c4, D):
     np.testing.assert_allclose(sums, 1.0, atol=1e-4)
 
 
+@pytest.mark.parametrize("D,shared", [(64, True), (16, True), (64, False)])
+def test_c4_fused_attention(c4, D, shared):
+    """Scores, softmax and weighted sum in one kernel on the whole 2.45M-vertex graph (hub rows of thousands of
+    edges included), against the three CPU checkers run one after the other; then with an all-ones value matrix,
+    where every row with an edge must come out as exactly the sum of its weights, 1."""
+    from featgraph_amd.module import MultiHeadAttentionhip
+    adj = c4
+    n, H = adj.shape[0], 8
+    _say("fused attention c4 H=8 D=%d %s through MultiHeadAttentionhip" % (D, "key = value" if shared else "key, value"))
+    module = MultiHeadAttentionhip(adj)
+    ph = [placeholder((n, H, D))] * (2 if shared else 3)
+    assert "fused" in module.lower_to_ir(ph, {}, {})
+    module.build(ph, {}, {})
+    key_dev, key = _device_normal((n, H, D), 800 + D, module.ctx)
+    key_dev *= 0.25
+    key *= np.float32(0.25)
+    query_dev, query = _device_normal((n, H, D), 900 + D, module.ctx)
+    ins, value = [key_dev, query_dev], None
+    if not shared:
+        value_dev, value = _device_normal((n, H, D), 950 + D, module.ctx)
+        ins.append(value_dev)
+    out = module.run(ins).asnumpy()
+    want = ref.attention_mh(adj.indptr, adj.indices, key, query, value)
+    np.testing.assert_allclose(out, want, rtol=1e-4, atol=1e-5)
+    del want, ins
+    if not shared:
+        value_dev.fill_(1.0)
+        out = module.run([key_dev, query_dev, value_dev]).asnumpy()
+        has_edges = np.diff(adj.indptr) > 0
+        np.testing.assert_allclose(out[has_edges], 1.0, rtol=2e-5)
+        assert not out[~has_edges].any()
+
+
 def test_benchmark_commands_run_on_a_small_graph(tmp_path, capsys):
     import scipy.sparse
     from featgraph_amd.benchmark import bench_vanilla_sddmm, bench_vanilla_spmm

@@ -345,3 +345,30 @@ def test_edge_softmax_against_scipy_and_its_invariants():
     uniform = ref.edge_softmax(adj.indptr, np.zeros((adj.nnz, H), np.float32))
     deg = np.repeat(np.diff(adj.indptr), np.diff(adj.indptr))
     np.testing.assert_allclose(uniform, (1.0 / deg)[:, None].repeat(H, 1), rtol=1e-6)
+
+
+def test_attention_against_dense_masked_softmax():
+    """The composed checker against the textbook dense form: softmax over a row's stored entries of Q K^T, times V
+    (float64 einsum on a matrix small enough to densify), with separate and with shared key / value."""
+    import scipy.special
+    rng = np.random.default_rng(11)
+    adj = scipy.sparse.random(37, 53, density=0.15, format="lil", random_state=rng)
+    adj[5] = 0
+    adj[36] = 0                                                              # rows without entries give zeros
+    adj = adj.tocsr()
+    adj.sort_indices()
+    H, D = 4, 8
+    key = rng.standard_normal((53, H, D), dtype=np.float32)
+    value = rng.standard_normal((53, H, D), dtype=np.float32)
+    query = rng.standard_normal((37, H, D), dtype=np.float32)
+    mask = adj.toarray() != 0
+    for val in (value, None):
+        v = key if val is None else val
+        scores = np.einsum("rhd,chd->hrc", query.astype(np.float64), key.astype(np.float64))
+        scores = np.where(mask[None], scores, -np.inf)
+        with np.errstate(invalid="ignore"):
+            weights = np.nan_to_num(scipy.special.softmax(scores, axis=2))    # rows without entries: all zero
+        want = np.einsum("hrc,chd->rhd", weights, v.astype(np.float64))
+        got = ref.attention_mh(adj.indptr, adj.indices, key, query, val)
+        np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
+    assert (np.diff(adj.indptr) == 0).any() and not got[np.diff(adj.indptr) == 0].any()
