@@ -30,6 +30,7 @@ between two events on the launch stream; the printed JSON line carries
 Only one GPU is used; --gpus above 1 is refused.
 """
 import argparse
+import ctypes
 import json
 import os
 import re
@@ -192,6 +193,23 @@ def main():
         return {"ms": ms, "row_bytes": row_floats * 4, "gathers": n_gathers,
                 "row_TBps": n_gathers * row_floats * 4 / ms / 1e9}
 
+    def rows_write_probe(feat_t, out_t, n_gathers, n_writes, read_only_ms, steps=3):
+        """Milliseconds for n_gathers random whole-row gathers from feat_t plus n_writes whole-row stores into out_t:
+        the read-only probe's rate for the gathers and, for the stores, the extra time per stored row that the
+        gather + store probe shows at (about) the same mix."""
+        n, row_floats = feat_t.shape[0], int(feat_t[0].numel())
+        g, w = ctypes.c_int64(0), ctypes.c_int64(0)
+        per = max(1, int(round(n_gathers / max(n_writes, 1))))
+        if L.fg_probe_gather_write_rows_count(row_floats, n_gathers, per, ctypes.byref(g), ctypes.byref(w)) != 0:
+            return None
+        ms = timed(lambda: _lib.check(L.fg_probe_gather_write_rows_f32(
+            feat_t.data_ptr(), n, row_floats, n_gathers, per, out_t.data_ptr(), out_t.shape[0], sink.data_ptr(),
+            stream.cuda_stream)), steps, 1)
+        per_gather = read_only_ms / n_gathers
+        per_write = max(0.0, (ms - g.value * per_gather) / max(w.value, 1))
+        return {"ms": n_gathers * per_gather + n_writes * per_write, "probe_ms": ms, "probe_gathers": g.value,
+                "probe_row_writes": w.value, "ms_per_million_row_writes": per_write * 1e6}
+
     if args.only == "copy":
         # plain device copy of known size: the yardstick the byte counters are scaled with
         n = 1 << 28
@@ -298,6 +316,14 @@ def main():
             else:
                 want = ref.spmm_mh(graph_adj.indptr, graph_adj.indices, w.cpu().numpy(), src.cpu().numpy())
                 row["parity"] = {"bit_exact_vs_cpu_checker": bool(np.array_equal(out, want))}
+        if p and kind in ("mh_spmm", "mh_attention", "mh_attention_kv"):
+            # these store one result row per destination row; the probe with stores in the same proportion (it
+            # overwrites the result, hence after the parity check) gives a ceiling that such an operator can reach
+            gathers = e * (2 if kind == "mh_attention_kv" else 1)
+            pw = rows_write_probe(src, op.out_tvm.tensor, gathers, n_r, p["ms"] * gathers / e)
+            if pw:
+                row.update({"gather_store_ceiling_ms": pw["ms"], "frac_of_gather_store_ceiling": pw["ms"] / ms,
+                            "gather_store_probe": pw})
         return row
 
     if args.only in ("mh_sddmm", "mh_spmm", "mh_sddmm_softmax", "mh_attention", "mh_attention_kv"):

@@ -53,16 +53,21 @@ __global__ __launch_bounds__(fg::kBlockThreads) void probe_gather_kernel(const f
 
 // Whole rows of `row_floats` floats (128, 256, or a multiple of 256) from anywhere in the matrix, addressed
 // in 64 bits: the pattern of the multi-head operators, whose feature matrices are far larger than any cache.
-// LPR lanes fetch one row with NV 16-byte loads each; 16 loads are in flight per lane.
+// LPR lanes fetch one row with NV 16-byte loads each; 16 loads are in flight per lane.  With write_every > 0
+// every group of LPR lanes also writes one whole row of `out` (a random one) after every write_every-th
+// iteration, as an operator that produces one result row per so many gathered rows does.
 template <int LPR, int NV>
 __global__ __launch_bounds__(fg::kBlockThreads) void probe_rows_kernel(const float *feat, int64_t row_floats,
-                                                                       uint32_t n_rows, int iters, float *sink) {
+                                                                       uint32_t n_rows, int iters, float *sink,
+                                                                       float *out, uint32_t out_rows,
+                                                                       int write_every) {
   constexpr int U = 16 / NV;
   const int lane = threadIdx.x & (fg::kWaveSize - 1);
   const int gl = lane & (LPR - 1), g = lane / LPR;
   const uint32_t wave = blockIdx.x * fg::kWavesPerBlock + (threadIdx.x >> 6);
   uint32_t s = wave * 2654435761u + static_cast<uint32_t>(g) * 40503u + 12345u;
   float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  int until_write = write_every;
   for (int it = 0; it < iters; ++it) {
     float4 x[U][NV];
 #pragma unroll
@@ -82,6 +87,13 @@ __global__ __launch_bounds__(fg::kBlockThreads) void probe_rows_kernel(const flo
         acc.z += x[u][k].z;
         acc.w += x[u][k].w;
       }
+    if (write_every > 0 && --until_write == 0) {
+      until_write = write_every;
+      const uint32_t r = (s >> 5) % out_rows;
+      float *q = out + static_cast<int64_t>(r) * row_floats + gl * 4;
+#pragma unroll
+      for (int k = 0; k < NV; ++k) *reinterpret_cast<float4 *>(q + k * 256) = acc;
+    }
   }
   if (acc.x + acc.y + acc.z + acc.w == __builtin_inff()) sink[0] = acc.x;
 }
@@ -104,8 +116,17 @@ bool rows_shape(int32_t row_floats, int *lpr, int *nv, int64_t *per_iter) {
 
 }  // namespace
 
-extern "C" int fg_probe_gather_rows_f32(const float *feat, int64_t n_rows, int32_t row_floats, int64_t n_gathers,
-                                        float *sink, void *stream) {
+// Iterations of the grid and, with writes, iterations between a group's writes, for a request.
+static int rows_iters(int64_t per_iter, int64_t n_gathers) {
+  return static_cast<int>(std::max<int64_t>(1, (n_gathers + per_iter / 2) / per_iter));
+}
+static int rows_write_every(int nv, int32_t gathers_per_write) {
+  const int u = 16 / nv;  // rows a group gathers per iteration
+  return gathers_per_write <= 0 ? 0 : std::max(1, (gathers_per_write + u / 2) / u);
+}
+
+static int probe_rows_run(const float *feat, int64_t n_rows, int32_t row_floats, int64_t n_gathers,
+                          int32_t gathers_per_write, float *out, int64_t n_out_rows, float *sink, void *stream) {
   if (!feat || !sink) return fg::fail(FG_EINVAL, "feat or sink is null");
   int lpr, nv;
   int64_t per_iter;
@@ -113,27 +134,56 @@ extern "C" int fg_probe_gather_rows_f32(const float *feat, int64_t n_rows, int32
     return fg::fail(FG_EINVAL, "row_floats = %d is not one of 128, 256, 512, 1024", row_floats);
   if (n_rows < 1 || n_rows > 0xffffffffLL || n_gathers < 0) return fg::fail(FG_EINVAL, "n_rows or n_gathers out of range");
   if (!fg::aligned_to(feat, 16)) return fg::fail(FG_EINVAL, "feat must be 16-byte aligned");
+  const int we = rows_write_every(nv, gathers_per_write);
+  if (we > 0 && (!out || n_out_rows < 1 || n_out_rows > 0xffffffffLL || !fg::aligned_to(out, 16)))
+    return fg::fail(FG_EINVAL, "writes need a 16-byte aligned out with 1 .. 2^32 - 1 rows");
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const int iters = static_cast<int>(std::max<int64_t>(1, (n_gathers + per_iter / 2) / per_iter));
-  const uint32_t n = static_cast<uint32_t>(n_rows);
+  const int iters = rows_iters(per_iter, n_gathers);
+  const uint32_t n = static_cast<uint32_t>(n_rows), no = static_cast<uint32_t>(we > 0 ? n_out_rows : 1);
   const dim3 grid(kProbeBlocks), block(fg::kBlockThreads);
   if (row_floats == 128)
-    probe_rows_kernel<32, 1><<<grid, block, 0, st>>>(feat, row_floats, n, iters, sink);
+    probe_rows_kernel<32, 1><<<grid, block, 0, st>>>(feat, row_floats, n, iters, sink, out, no, we);
   else if (row_floats == 256)
-    probe_rows_kernel<64, 1><<<grid, block, 0, st>>>(feat, row_floats, n, iters, sink);
+    probe_rows_kernel<64, 1><<<grid, block, 0, st>>>(feat, row_floats, n, iters, sink, out, no, we);
   else if (row_floats == 512)
-    probe_rows_kernel<64, 2><<<grid, block, 0, st>>>(feat, row_floats, n, iters, sink);
+    probe_rows_kernel<64, 2><<<grid, block, 0, st>>>(feat, row_floats, n, iters, sink, out, no, we);
   else
-    probe_rows_kernel<64, 4><<<grid, block, 0, st>>>(feat, row_floats, n, iters, sink);
+    probe_rows_kernel<64, 4><<<grid, block, 0, st>>>(feat, row_floats, n, iters, sink, out, no, we);
   FG_HIP_TRY(hipGetLastError());
   return FG_OK;
+}
+
+extern "C" int fg_probe_gather_rows_f32(const float *feat, int64_t n_rows, int32_t row_floats, int64_t n_gathers,
+                                        float *sink, void *stream) {
+  return probe_rows_run(feat, n_rows, row_floats, n_gathers, 0, nullptr, 0, sink, stream);
 }
 
 extern "C" int64_t fg_probe_gather_rows_count(int32_t row_floats, int64_t n_gathers) {
   int lpr, nv;
   int64_t per_iter;
   if (!rows_shape(row_floats, &lpr, &nv, &per_iter) || n_gathers < 0) return -1;
-  return std::max<int64_t>(1, (n_gathers + per_iter / 2) / per_iter) * per_iter;
+  return rows_iters(per_iter, n_gathers) * per_iter;
+}
+
+extern "C" int fg_probe_gather_write_rows_f32(const float *feat, int64_t n_rows, int32_t row_floats,
+                                              int64_t n_gathers, int32_t gathers_per_write, float *out,
+                                              int64_t n_out_rows, float *sink, void *stream) {
+  if (gathers_per_write < 1) return fg::fail(FG_EINVAL, "gathers_per_write = %d must be positive", gathers_per_write);
+  return probe_rows_run(feat, n_rows, row_floats, n_gathers, gathers_per_write, out, n_out_rows, sink, stream);
+}
+
+extern "C" int fg_probe_gather_write_rows_count(int32_t row_floats, int64_t n_gathers, int32_t gathers_per_write,
+                                                int64_t *gathers, int64_t *writes) {
+  int lpr, nv;
+  int64_t per_iter;
+  if (!gathers || !writes) return fg::fail(FG_EINVAL, "a result pointer is null");
+  if (!rows_shape(row_floats, &lpr, &nv, &per_iter) || n_gathers < 0 || gathers_per_write < 1)
+    return fg::fail(FG_EINVAL, "row_floats, n_gathers or gathers_per_write out of range");
+  const int iters = rows_iters(per_iter, n_gathers);
+  const int64_t groups = int64_t{kProbeBlocks} * fg::kWavesPerBlock * (fg::kWaveSize / lpr);
+  *gathers = iters * per_iter;
+  *writes = groups * (iters / rows_write_every(nv, gathers_per_write));
+  return FG_OK;
 }
 
 extern "C" int fg_probe_gather_f32(const float *feat, int64_t n_rows, int32_t F, int32_t tile, int32_t band_rows,

@@ -302,6 +302,21 @@ FG_API int64_t fg_probe_gather_count(int64_t n_rows, int32_t tile, int32_t band_
 FG_API int fg_probe_gather_rows_f32(const float *feat, int64_t n_rows, int32_t row_floats, int64_t n_gathers,
                                     float *sink, void *stream);
 FG_API int64_t fg_probe_gather_rows_count(int32_t row_floats, int64_t n_gathers);
+/*
+ * The same with result rows: after about every gathers_per_write gathered rows
+ * (rounded to whole iterations of 16 / 8 / 4 rows for rows of up to 256 / 512 /
+ * 1024 floats) a group of lanes also writes one whole row of out
+ * [n_out_rows, row_floats], a random one.  An operator that gathers deg rows
+ * and stores one per destination row moves this mix; on this part the stores
+ * cost several times their share of the bytes, so the read-only probe is not a
+ * floor such an operator can reach.  fg_probe_gather_write_rows_count gives the
+ * gathers and the row writes that a call with these arguments issues.
+ */
+FG_API int fg_probe_gather_write_rows_f32(const float *feat, int64_t n_rows, int32_t row_floats, int64_t n_gathers,
+                                          int32_t gathers_per_write, float *out, int64_t n_out_rows, float *sink,
+                                          void *stream);
+FG_API int fg_probe_gather_write_rows_count(int32_t row_floats, int64_t n_gathers, int32_t gathers_per_write,
+                                            int64_t *gathers, int64_t *writes);
 
 /*
  * Launch-shape overrides for tuning and tests.  The store is process-global

@@ -109,3 +109,10 @@ def test_error_codes_of_the_later_entry_points_without_a_device():
     assert L.fg_probe_gather_count(232965, 64, 16384, 114606755) >= 100_000_000
     assert L.fg_probe_gather_rows_f32(8, 4, 100, 10, 8, None) == -1
     assert L.fg_probe_gather_rows_count(512, 61948164) >= 60_000_000
+    assert L.fg_probe_gather_write_rows_f32(16, 4, 512, 10, 0, 16, 4, 16, None) == -1    # a write per 0 gathers
+    assert L.fg_probe_gather_write_rows_f32(16, 4, 512, 10, 24, None, 4, 16, None) == -1  # no result matrix
+    g, w = ctypes.c_int64(0), ctypes.c_int64(0)
+    assert L.fg_probe_gather_write_rows_count(512, 61948164, 25, ctypes.byref(g), ctypes.byref(w)) == 0
+    assert g.value >= 60_000_000 and 20 <= g.value / w.value <= 30                        # about one write per 25 gathers
+    assert L.fg_probe_gather_write_rows_count(100, 10, 25, ctypes.byref(g), ctypes.byref(w)) == -1
+    assert L.fg_attention_csr_mh_f32(None, None, None, None, None, 8, 64, None) == -1
