@@ -47,6 +47,9 @@ struct fg_spmm_plan {
   int32_t *seg;  // owned, device, (n_blocks + 1) * n_rows entries
   int32_t n_blocks;
   int32_t block_cols;
+  // When the library sizes the blocks it may cut each block of the default width into `split` equal ones, so
+  // that a kernel can take 1 .. split neighbouring blocks per pass; split_used is 1 when the caller sized them.
+  int32_t split = 1, split_used = 1;
   int32_t requested_partitions;  // 0: library decides; 1: no column blocks; P > 1: P blocks, as the caller asked
   bool force_blocks;             // the caller's P > 1: use the blocks at every feature length
   // what the bounds table is built from: block width (0: default), blocks on / off / automatic (1 / 0 / -1),
@@ -76,7 +79,8 @@ struct fg_sddmm_plan {
 
 static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr, const int32_t *indices,
                            int32_t num_col_partitions, int32_t want_block_cols, int32_t default_block_cols,
-                           int want_blocked, double min_per_segment, bool with_multi, fg_spmm_plan **plan);
+                           int32_t split, int want_blocked, double min_per_segment, bool with_multi,
+                           fg_spmm_plan **plan);
 
 namespace {
 
@@ -150,6 +154,9 @@ int check_device(int plan_device) {
 // 12 passes of 19,414 columns 1.86 ms, 15 of 15,532 1.95 ms, 9 of 25,885 1.98 ms).
 constexpr int32_t kSpmmBlockCols = 20480;
 constexpr int32_t kSddmmBlockCols = 16384;
+// The SDDMM row plan cuts each of those blocks in two: a pass of the row-run kernel takes both halves for a
+// 64-float tile and one for a 128-float tile, so the band it gathers from stays 4 MB.
+constexpr int32_t kSddmmSplit = 2;
 
 int check_heads(int32_t H, int32_t D) {
   if (H < 1 || D < 1) return fg::fail(FG_EINVAL, "H = %d and D = %d must both be positive", H, D);
@@ -342,10 +349,16 @@ int build_bounds(fg_spmm_plan *p) {
   const int P = p->requested_partitions;
   if (P > 1) block_cols = std::max<int64_t>(1, (p->n_cols + P - 1) / P);  // util/adj_partitioning.py:42
   int64_t n_blocks = p->n_cols > 0 ? (p->n_cols + block_cols - 1) / block_cols : 1;
-  // the library's own blocks: as many as the default width asks for, all of the same width
-  if (P <= 1 && p->want_block_cols <= 0 && n_blocks > 1) block_cols = (p->n_cols + n_blocks - 1) / n_blocks;
+  // whether blocks pay is judged at the default width, before any split
   const double per_segment =
       n_blocks > 0 ? static_cast<double>(p->nnz) / (static_cast<double>(p->n_rows) * n_blocks) : 0.0;
+  // the library's own blocks: as many as the default width asks for (times the split), all of the same width
+  p->split_used = 1;
+  if (P <= 1 && p->want_block_cols <= 0 && n_blocks > 1) {
+    p->split_used = std::max(1, p->split);
+    n_blocks *= p->split_used;
+    block_cols = (p->n_cols + n_blocks - 1) / n_blocks;
+  }
   if (P == 1 || n_blocks < 2 || p->nnz == 0)
     n_blocks = 1;
   else if (P == 0 && (p->want_blocked == 0 || (p->want_blocked < 0 && per_segment < p->min_per_segment)))
@@ -354,7 +367,7 @@ int build_bounds(fg_spmm_plan *p) {
   int *flag = nullptr;
   FG_HIP_TRY(hipMalloc(&flag, sizeof(int)));
   for (;;) {
-    if (n_blocks == 1) block_cols = 0x7fffffff;
+    if (n_blocks == 1) block_cols = 0x7fffffff, p->split_used = 1;
     int32_t *seg = nullptr;
     hipError_t err = hipMalloc(&seg, static_cast<size_t>(n_blocks + 1) * p->n_rows * sizeof(int32_t));
     if (err == hipErrorOutOfMemory && n_blocks > 1) {  // no room for the blocks: whole rows only
@@ -417,6 +430,7 @@ int *config_slot(const char *key) {
   if (!strcmp(key, "sddmm.buffer_loads")) return &c.sddmm_buffer_loads;
   if (!strcmp(key, "sddmm.rows")) return &c.sddmm_rows;
   if (!strcmp(key, "sddmm.rows_blocks")) return &c.sddmm_rows_blocks;
+  if (!strcmp(key, "sddmm.rows_wide")) return &c.sddmm_rows_wide;
   if (!strcmp(key, "attention.blocks")) return &c.attention_blocks;
   return nullptr;
 }
@@ -459,14 +473,15 @@ int fg_spmm_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32
 int fg_spmm_plan_create_partitioned(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr,
                                     const int32_t *indices, int32_t num_col_partitions, fg_spmm_plan **plan) {
   return row_plan_create(n_rows, n_cols, nnz, indptr, indices, num_col_partitions, fg::config().spmm_block_cols,
-                         kSpmmBlockCols, fg::config().spmm_blocked, 8.0, true, plan);
+                         kSpmmBlockCols, 1, fg::config().spmm_blocked, 8.0, true, plan);
 }
 
 // want_block_cols / want_blocked / min_per_segment: see fg_spmm_plan; with_multi: also build the records of the
 // several-rows-per-wave kernel.
 static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr, const int32_t *indices,
                            int32_t num_col_partitions, int32_t want_block_cols, int32_t default_block_cols,
-                           int want_blocked, double min_per_segment, bool with_multi, fg_spmm_plan **plan) {
+                           int32_t split, int want_blocked, double min_per_segment, bool with_multi,
+                           fg_spmm_plan **plan) {
   if (!plan) return fg::fail(FG_EINVAL, "plan output pointer is null");
   *plan = nullptr;
   if (num_col_partitions < 0)
@@ -517,6 +532,7 @@ static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const in
   p->force_blocks = false;
   p->want_block_cols = want_block_cols;
   p->default_block_cols = default_block_cols;
+  p->split = split;
   p->want_blocked = want_blocked;
   p->min_per_segment = min_per_segment;
   p->max_degree = max_degree;
@@ -661,8 +677,8 @@ static int build_row_runs(fg_sddmm_plan *p, int32_t num_col_partitions) {
   // same block width as the re-ordered edge list (sddmm_blocked.hip); a run costs a wave a fixed amount of
   // work, so blocks need 8 edges per run on average (sparser lists keep whole rows and take the edge-list path)
   return row_plan_create(p->n_rows, p->n_cols, p->nnz, p->indptr, p->col, num_col_partitions,
-                         fg::config().sddmm_block_cols, kSddmmBlockCols, fg::config().sddmm_blocked, 8.0, false,
-                         &p->rows);
+                         fg::config().sddmm_block_cols, kSddmmBlockCols, kSddmmSplit, fg::config().sddmm_blocked, 8.0,
+                         false, &p->rows);
 }
 
 int fg_sddmm_plan_create(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,
@@ -724,13 +740,26 @@ static bool sddmm_use_blocks(const fg_sddmm_plan *plan, const float *src, const 
          fg::aligned_to(dst, 16);
 }
 
-// Column blocks of the table that one pass of the row-run kernel takes together: the band of Src that a pass
-// gathers from (block width x tile bytes) should stay about one L2 (4 MB), so narrower tiles take wider
-// blocks.  Blocks that the caller sized (partition count, sddmm.block_cols) are used as they are.
-static int sddmm_rows_merge(const fg_sddmm_plan *plan, int32_t D) {
+// Column blocks of the table that one pass of the row-run kernel takes together for a 64-float tile: the band
+// of Src that a pass gathers from (block width x tile bytes) should stay about one L2 (4 MB), so narrower
+// tiles take more blocks and wider tiles fewer.  Blocks that the caller sized (partition count,
+// sddmm.block_cols) are used as they are.
+static int sddmm_rows_merge64(const fg_sddmm_plan *plan) {
   const fg_spmm_plan *r = plan->rows;
-  if (plan->force_blocks || r->want_block_cols > 0 || r->n_blocks < 2) return 1;
-  return 64 / fg::sddmm_rows_tile(D);  // the table's blocks are sized for 64-float tiles
+  if (plan->force_blocks || r->want_block_cols > 0 || r->n_blocks < 2) return 0;  // 0: one block per pass, always
+  return r->split_used;
+}
+
+// Widest tile, in 64-float units (1 or 2), that the row-run kernel may use: the passes of a wider tile are
+// narrower by the same factor, and a (row, pass) run should still hold 8 edges on average.
+static int sddmm_rows_max_wide(const fg_sddmm_plan *plan) {
+  const fg_spmm_plan *r = plan->rows;
+  const int merge64 = sddmm_rows_merge64(plan);
+  const int want = fg::config().sddmm_rows_wide;
+  if (want > 0) return want >= 2 ? 2 : 1;  // asked for: also over blocks that the caller sized (their width stays)
+  if (merge64 == 0 || merge64 % 2 != 0) return 1;
+  const double per_block = static_cast<double>(plan->nnz) / (static_cast<double>(r->n_rows) * r->n_blocks);
+  return per_block * (merge64 / 2) >= 8.0 ? 2 : 1;
 }
 
 static bool sddmm_use_row_runs(const fg_sddmm_plan *plan, const float *src, const float *dst, int32_t H, int32_t D) {
@@ -754,7 +783,7 @@ int fg_sddmm_coo_plan_f32(const fg_sddmm_plan *plan, const float *src, const flo
     if (!src || !dst || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
     const fg_spmm_plan *r = plan->rows;
     return fg::sddmm_rows_launch(r->seg, r->row_order, static_cast<int32_t>(r->n_rows), r->n_blocks,
-                                 sddmm_rows_merge(plan, D), plan->col, src,
+                                 sddmm_rows_merge64(plan), sddmm_rows_max_wide(plan), plan->col, src,
                                  dst, out, plan->n_cols * int64_t{D} * 4, plan->n_rows * int64_t{D} * 4, D,
                                  static_cast<hipStream_t>(stream));
   }
@@ -819,16 +848,18 @@ int fg_sddmm_plan_describe(const fg_sddmm_plan *plan, int32_t H, int32_t D, char
   if (!buf || cap <= 0) return fg::fail(FG_EINVAL, "no room for the description");
   alignas(16) static float dummy[4];
   if (sddmm_use_row_runs(plan, dummy, dummy, H, D)) {
-    const int rows_tile = fg::sddmm_rows_tile(D);
-    const int merge = sddmm_rows_merge(plan, D);
+    // the first launch's tile (later launches of a long feature row may take a narrower rest)
+    const int rows_tile = fg::sddmm_rows_tile(D, sddmm_rows_max_wide(plan));
+    const int merge64 = sddmm_rows_merge64(plan);
+    const int merge = merge64 == 0 ? 1 : rows_tile <= 64 ? merge64 * (64 / rows_tile) : std::max(1, merge64 / (rows_tile / 64));
     snprintf(buf, static_cast<size_t>(cap),
              "sddmm_coo nnz=%lld H=%d D=%d | kernel=row runs (row-sorted edge list), %d column blocks of %d, tile=%d "
-             "floats x %d tiles (one launch each), floats/lane=4 lanes/dot=%d | grid=(blocks, column blocks) x %d "
+             "floats x %d tiles (one launch each), floats/lane=%d lanes/dot=%d | grid=(blocks, column blocks) x %d "
              "threads each",
              (long long)plan->nnz, H, D, (plan->rows->n_blocks + merge - 1) / merge,
              static_cast<int>(std::min<int64_t>(int64_t{plan->rows->block_cols} * merge, 0x7fffffff)), rows_tile,
-             (D + rows_tile - 1) / rows_tile,
-             rows_tile / 4, fg::kBlockThreads);
+             (D + rows_tile - 1) / rows_tile, rows_tile <= 64 ? 4 : rows_tile / 16, std::min(rows_tile / 4, 16),
+             fg::kBlockThreads);
     return FG_OK;
   }
   if (!sddmm_use_blocks(plan, dummy, dummy, H, D)) return fg_sddmm_describe(plan->nnz, H, D, buf, cap);

@@ -28,7 +28,7 @@ struct Config {
   int spmm_multi = -1, spmm_multi_blocks = 0, spmm_multi_long = 0, spmm_tile_interleave = 0;
   int sddmm_group = 0, sddmm_batches = 0, sddmm_blocked = -1, sddmm_block_cols = 0;
   int sddmm_fast = -1, sddmm_buffer_loads = -1, sddmm_rows = -1, sddmm_rows_blocks = 0;
-  int attention_blocks = 0;
+  int attention_blocks = 0, sddmm_rows_wide = 0;
 };
 Config &config();
 
@@ -139,13 +139,16 @@ int sddmm_tile_launch(const int32_t *row_p, const int32_t *col_p, const int32_t 
                       const float *dst, float *out, int64_t src_bytes, int64_t dst_bytes, int32_t F, int tile,
                       hipStream_t stream);
 
-// Row-run kernel over (column block, row) runs of a row-sorted edge list: one launch per tile of
-// sddmm_rows_tile(F) floats, grid.y = column block.  seg / row_order are the bounds table and row list of a
-// row plan built on the same matrix; `merge` neighbouring blocks of the table are taken as one (sddmm.hip).
-int sddmm_rows_tile(int32_t F);
-int sddmm_rows_launch(const int32_t *seg, const int32_t *row_order, int32_t n_rows, int32_t n_blocks, int32_t merge,
-                      const int32_t *col, const float *src, const float *dst, float *out, int64_t src_bytes,
-                      int64_t dst_bytes, int32_t F, hipStream_t stream);
+// Row-run kernel over (column block, row) runs of a row-sorted edge list: one launch per tile, grid.y = column
+// block.  A tile is sddmm_rows_tile(F, max_wide) floats: 16 / 32 / 64 for short rows, and max_wide (1 or 2)
+// times 64 for longer ones.  seg / row_order are the bounds table and row list of a row plan built on the
+// same matrix; a pass of a 64-float tile takes merge64 neighbouring blocks of the table, narrower tiles
+// proportionally more, wider tiles proportionally fewer; merge64 = 0 means one block per pass for every tile
+// (sddmm.hip).
+int sddmm_rows_tile(int32_t F, int max_wide);
+int sddmm_rows_launch(const int32_t *seg, const int32_t *row_order, int32_t n_rows, int32_t n_blocks, int32_t merge64,
+                      int max_wide, const int32_t *col, const float *src, const float *dst, float *out,
+                      int64_t src_bytes, int64_t dst_bytes, int32_t F, hipStream_t stream);
 
 // Generalised operators (general.hip): msg / reduce / op are the FG_MSG_* / FG_REDUCE_* / FG_EDGE_* codes.
 int spmm_general_launch(const int32_t *row_order, const int32_t *seg_lo, const int32_t *seg_hi, const int32_t *indices,

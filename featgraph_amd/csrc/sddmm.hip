@@ -246,9 +246,11 @@ struct RowsArgs {
   int32_t n_blocks, merge;   // column blocks in the table; blockIdx.y covers `merge` neighbouring ones
 };
 
-// G: lanes per dot product (a tile is 4 * G floats); R: rounds whose gathers are issued together.
-template <bool ACC, bool BUF, int R, int G>
+// G: lanes per dot product; NT: 16-byte pieces per lane, 64 floats apart (a tile is 4 * G * NT floats; NT > 1
+// needs G = 16); R: rounds whose gathers are issued together.
+template <bool ACC, bool BUF, int R, int G, int NT>
 __global__ __launch_bounds__(kBlockThreads) void sddmm_rows_kernel(const RowsArgs a) {
+  static_assert(NT == 1 || G == 16, "a wide tile is made of whole 64-float pieces");
   constexpr int NG = kWaveSize / G;  // edges per round
   const int lane = threadIdx.x & (kWaveSize - 1);
   const int gl = lane & (G - 1);
@@ -260,8 +262,15 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_rows_kernel(const RowsArg
   const int32_t *const seg_hi = a.seg + static_cast<int64_t>(min((blockIdx.y + 1) * a.merge, a.n_blocks)) * n;
   const VertexRows<BUF> src(a.src, a.src_bytes), dst(a.dst, a.dst_bytes);
   const uint32_t row_bytes = static_cast<uint32_t>(a.F) * 4u;
-  const bool kok = gl * 4 < a.valid;
-  const uint32_t lane_bytes = static_cast<uint32_t>(a.first + (kok ? gl * 4 : a.valid - 4)) * 4u;
+  // piece k of this lane covers floats first + 64 k + 4 gl ..; lanes past the tile's end re-read its last
+  // four floats and contribute zero
+  bool kok[NT];
+  uint32_t lane_bytes[NT];
+#pragma unroll
+  for (int k = 0; k < NT; ++k) {
+    kok[k] = k * 64 + gl * 4 < a.valid;
+    lane_bytes[k] = static_cast<uint32_t>(a.first + (kok[k] ? k * 64 + gl * 4 : a.valid - 4)) * 4u;
+  }
   const int gather_from = G * (lane % NG) + lane / NG;  // lane holding the result of edge offset `lane`
 
   auto bounds = [&](int it, int &lo, int &hi, int &row) {
@@ -272,21 +281,23 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_rows_kernel(const RowsArg
       row = a.row_order[it];
     }
   };
-  auto first_block = [&](int lo, int hi, int row, int &col, float4 &y, float &prev) {
+  auto first_block = [&](int lo, int hi, int row, int &col, float4(&y)[NT], float &prev) {
     col = 0;
     prev = 0.0f;
-    y = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+    for (int k = 0; k < NT; ++k) y[k] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     if (hi > lo) {
       if (lane < hi - lo) {
         col = a.col[lo + lane];
         if (ACC) prev = a.out[lo + lane];
       }
-      y = dst.load(row, row_bytes, lane_bytes);
+#pragma unroll
+      for (int k = 0; k < NT; ++k) y[k] = dst.load(row, row_bytes, lane_bytes[k]);
     }
   };
 
   int lo_a, hi_a, row_a, col_a, lo_b, hi_b, row_b;
-  float4 y_a;
+  float4 y_a[NT];
   float prev_a;
   bounds(item, lo_a, hi_a, row_a);
   first_block(lo_a, hi_a, row_a, col_a, y_a, prev_a);
@@ -294,7 +305,9 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_rows_kernel(const RowsArg
 
   while (item < n) {
     int lo_c, hi_c, row_c, col_b = 0;
-    float4 y_b = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    float4 y_b[NT];
+#pragma unroll
+    for (int k = 0; k < NT; ++k) y_b[k] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     float prev_b = 0.0f;
     bounds(item + 2 * n_waves, lo_c, hi_c, row_c);
     bool next_asked = false;
@@ -310,24 +323,29 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_rows_kernel(const RowsArg
       const int rounds = (cnt + NG - 1) / NG;
       float res = 0.0f;
       // two batches of R rounds alternate: the gathers of one are in flight while the other is summed
-      float4 xa[R], xb[R];
-      auto issue = [&](int rb, float4(&x)[R]) {
+      float4 xa[R][NT], xb[R][NT];
+      auto issue = [&](int rb, float4(&x)[R][NT]) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           // edges past the run's end read column id 0 of an idle lane: a valid row, result never stored
           const int cc = __builtin_amdgcn_ds_bpermute(((NG * (rb + r) + g) & 63) << 2, col_a);
-          x[r] = src.load(cc, row_bytes, lane_bytes);
+#pragma unroll
+          for (int k = 0; k < NT; ++k) x[r][k] = src.load(cc, row_bytes, lane_bytes[k]);
         }
       };
-      auto reduce = [&](int rb, const float4(&x)[R]) {
+      auto reduce = [&](int rb, const float4(&x)[R][NT]) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           float p = 0.0f;
-          p = __builtin_fmaf(x[r].x, y_a.x, p);
-          p = __builtin_fmaf(x[r].y, y_a.y, p);
-          p = __builtin_fmaf(x[r].z, y_a.z, p);
-          p = __builtin_fmaf(x[r].w, y_a.w, p);
-          p = kok ? p : 0.0f;
+#pragma unroll
+          for (int k = 0; k < NT; ++k) {
+            float q = 0.0f;
+            q = __builtin_fmaf(x[r][k].x, y_a[k].x, q);
+            q = __builtin_fmaf(x[r][k].y, y_a[k].y, q);
+            q = __builtin_fmaf(x[r][k].z, y_a[k].z, q);
+            q = __builtin_fmaf(x[r][k].w, y_a[k].w, q);
+            p += kok[k] ? q : 0.0f;
+          }
           p = group_sum<G>(p);
           if (gl == rb + r) res = p;
         }
@@ -359,7 +377,8 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_rows_kernel(const RowsArg
     hi_a = hi_b;
     row_a = row_b;
     col_a = col_b;
-    y_a = y_b;
+#pragma unroll
+    for (int k = 0; k < NT; ++k) y_a[k] = y_b[k];
     prev_a = prev_b;
     lo_b = lo_c;
     hi_b = hi_c;
@@ -463,26 +482,35 @@ int sddmm_tile_launch(const int32_t *row_p, const int32_t *col_p, const int32_t 
   return tile == 0 ? launch_fast_mode<16, 1, false, 1>(f, stream) : launch_fast_mode<16, 1, false, 2>(f, stream);
 }
 
-template <int G>
+template <int G, int NT>
 static void rows_dispatch(const RowsArgs &a, bool acc, bool buf, dim3 grid, hipStream_t stream) {
+  constexpr int R = NT == 2 ? 1 : 2;  // rounds per batch: four 16-byte gathers in flight per lane, two batches
   if (!acc) {
     if (buf)
-      sddmm_rows_kernel<false, true, 2, G><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+      sddmm_rows_kernel<false, true, R, G, NT><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
     else
-      sddmm_rows_kernel<false, false, 2, G><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+      sddmm_rows_kernel<false, false, R, G, NT><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
   } else {
     if (buf)
-      sddmm_rows_kernel<true, true, 2, G><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+      sddmm_rows_kernel<true, true, R, G, NT><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
     else
-      sddmm_rows_kernel<true, false, 2, G><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+      sddmm_rows_kernel<true, false, R, G, NT><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
   }
 }
 
-int sddmm_rows_tile(int32_t F) { return F <= 16 ? 16 : F <= 32 ? 32 : 64; }
+// Width of the (first) tile: the whole row when it is short (then fewer lanes share a dot product), else 64
+// floats, or 128 when wide tiles are allowed and the row has that many left.  (256-float tiles over passes of
+// a quarter of the width measured slower: 8.6 against 7.7 ms at 256 floats on the 114.6M-edge benchmark graph.)
+int sddmm_rows_tile(int32_t F, int max_wide) {
+  if (F <= 16) return 16;
+  if (F <= 32) return 32;
+  if (max_wide >= 2 && F >= 128) return 128;
+  return 64;
+}
 
-int sddmm_rows_launch(const int32_t *seg, const int32_t *row_order, int32_t n_rows, int32_t n_blocks, int32_t merge,
-                      const int32_t *col, const float *src, const float *dst, float *out, int64_t src_bytes,
-                      int64_t dst_bytes, int32_t F, hipStream_t stream) {
+int sddmm_rows_launch(const int32_t *seg, const int32_t *row_order, int32_t n_rows, int32_t n_blocks, int32_t merge64,
+                      int max_wide, const int32_t *col, const float *src, const float *dst, float *out,
+                      int64_t src_bytes, int64_t dst_bytes, int32_t F, hipStream_t stream) {
   if (n_rows == 0) return FG_OK;
   RowsArgs a;
   a.seg = seg;
@@ -497,25 +525,30 @@ int sddmm_rows_launch(const int32_t *seg, const int32_t *row_order, int32_t n_ro
   a.F = F;
   int64_t blocks = config().sddmm_rows_blocks > 0 ? config().sddmm_rows_blocks : 16384;
   blocks = std::max<int64_t>(1, std::min<int64_t>(blocks, (n_rows + kWavesPerBlock - 1) / kWavesPerBlock));
-  merge = std::max(1, std::min(merge, n_blocks));
   a.n_blocks = n_blocks;
-  a.merge = merge;
-  const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>((n_blocks + merge - 1) / merge));
   const bool buf = src_bytes < (int64_t{1} << 32) && dst_bytes < (int64_t{1} << 32) && config().sddmm_buffer_loads != 0;
-  // tile width: 64 floats, or the whole row when it is shorter (then fewer lanes share a dot product)
-  const int tile = sddmm_rows_tile(F);
-  const int G = tile / 4;
-  const int n_tiles = (F + tile - 1) / tile;
-  for (int t = 0; t < n_tiles; ++t) {
-    a.first = t * tile;
-    a.valid = std::min(F - t * tile, tile);
-    if (G == 4)
-      rows_dispatch<4>(a, t > 0, buf, grid, stream);
-    else if (G == 8)
-      rows_dispatch<8>(a, t > 0, buf, grid, stream);
+  // One launch per tile; every launch after the first adds to the partial dot products that the one before
+  // left in Out.  A long row is cut into the widest tiles allowed, its rest into narrower ones.
+  for (int first = 0; first < F;) {
+    const int tile = sddmm_rows_tile(F - first, max_wide);
+    // the band a pass gathers from keeps its size: wider tiles take fewer of the table's blocks per pass
+    // (merge64 = 0: the caller sized the blocks, one per pass whatever the tile)
+    const int merge = std::max(1, std::min(tile <= 64 ? merge64 * (64 / tile) : merge64 / (tile / 64), n_blocks));
+    a.merge = merge;
+    a.first = first;
+    a.valid = std::min(F - first, tile);
+    const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>((n_blocks + merge - 1) / merge));
+    const bool acc = first > 0;
+    if (tile == 16)
+      rows_dispatch<4, 1>(a, acc, buf, grid, stream);
+    else if (tile == 32)
+      rows_dispatch<8, 1>(a, acc, buf, grid, stream);
+    else if (tile == 64)
+      rows_dispatch<16, 1>(a, acc, buf, grid, stream);
     else
-      rows_dispatch<16>(a, t > 0, buf, grid, stream);
+      rows_dispatch<16, 2>(a, acc, buf, grid, stream);
     FG_HIP_TRY(hipGetLastError());
+    first += a.valid;
   }
   return FG_OK;
 }

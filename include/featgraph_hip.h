@@ -348,6 +348,9 @@ FG_API int fg_probe_gather_write_rows_count(int32_t row_floats, int64_t n_gather
  * kernel for D in 16..512), "sddmm.buffer_loads" (0/1), "sddmm.rows" (0/1:
  * never / always use the row-run kernel when the plan has a row plan; read at
  * plan creation and at launch), "sddmm.rows_blocks" (its grid size),
+ * "sddmm.rows_wide" (1: 64-float tiles only, 2: 128-float tiles over passes of
+ * half the width for feature rows of 128 floats and more; by default 2 when a
+ * (row, pass) run then still holds 8 edges on average),
  * "attention.blocks" (grid size of the fused attention kernel).  Value 0 restores the default of
  * a size; for the 0/1 flags a negative value does.
  * The spmm.* keys change the launch shape only; "sddmm.group" also changes the

@@ -32,6 +32,7 @@ def config_guard():
     _lib.config_set("sddmm.batches", 0)
     _lib.config_set("sddmm.block_cols", 0)
     _lib.config_set("sddmm.rows_blocks", 0)
+    _lib.config_set("sddmm.rows_wide", 0)
     for key in ("sddmm.blocked", "sddmm.fast", "sddmm.buffer_loads", "sddmm.rows"):
         _lib.config_set(key, -1)
 
@@ -234,6 +235,30 @@ def test_row_runs_of_a_row_sorted_list(config_guard, F):
     module = VanillaSDDMMhip(coo)
     assert "column-blocked edge list" in _describe(module, src, dst)
     assert np.array_equal(_run_sddmm(coo, src, dst), outs[0])
+
+
+@pytest.mark.parametrize("F", [128, 132, 192, 200, 260, 512])
+def test_row_runs_with_tiles_of_128_floats(config_guard, F):
+    """Feature rows of 128 floats and more go through 128-float tiles (two 16-byte pieces per lane), the rest of a
+    row through narrower ones; same results as 64-float tiles within the tolerance (the summation tree differs)."""
+    coo = datasets.config_graph("c2-mini").tocoo()
+    src, dst = datasets.sddmm_operands(coo, F)
+    exact = ref.sddmm_f64(coo.row, coo.col, src, dst)
+    _lib.config_set("sddmm.blocked", 1)
+    _lib.config_set("sddmm.block_cols", 700)
+    outs = {}
+    for wide in (1, 2):
+        _lib.config_set("sddmm.rows_wide", wide)
+        module = VanillaSDDMMhip(coo)
+        text = _describe(module, src, dst)
+        assert "row runs" in text and "tile=%d floats" % (64 * wide) in text
+        module.build([placeholder(src.shape), placeholder(dst.shape)], {}, {})
+        module.out_tvm.tensor.fill_(7.0)
+        outs[wide] = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
+        np.testing.assert_allclose(outs[wide], exact, rtol=RTOL, atol=ATOL)
+    isrc, idst = np.rint(src * 2), np.rint(dst * 2)                  # small integers: every order gives the same sum
+    _lib.config_set("sddmm.rows_wide", 2)
+    assert np.array_equal(_run_sddmm(coo, isrc, idst), ref.sddmm_f64(coo.row, coo.col, isrc, idst).astype(np.float32))
 
 
 def test_row_runs_only_for_row_sorted_lists(config_guard):
