@@ -275,6 +275,8 @@ def main():
             b, b_min = mh_spmm_alg_bytes(e, n_r, H, D), 4 * e + 4 * H * e + 4 * (n_r + 1) + 4 * H * D * (n_r + n_c)
         ms = timed(lambda: op.run(ins), steps, warmup)
         p = rows_probe(src, e)
+        if p and kind == "mh_attention_kv":      # two gathered rows per edge
+            p = dict(p, ms=2 * p["ms"], gathers=2 * e)
         if p:
             row.update({"gather_ceiling_ms": p["ms"], "gather_ceiling_row_TBps": p["row_TBps"],
                         "frac_of_gather_ceiling": p["ms"] / ms})
@@ -320,7 +322,7 @@ def main():
             # these store one result row per destination row; the probe with stores in the same proportion (it
             # overwrites the result, hence after the parity check) gives a ceiling that such an operator can reach
             gathers = e * (2 if kind == "mh_attention_kv" else 1)
-            pw = rows_write_probe(src, op.out_tvm.tensor, gathers, n_r, p["ms"] * gathers / e)
+            pw = rows_write_probe(src, op.out_tvm.tensor, gathers, n_r, p["ms"])
             if pw:
                 row.update({"gather_store_ceiling_ms": pw["ms"], "frac_of_gather_store_ceiling": pw["ms"] / ms,
                             "gather_store_probe": pw})
