@@ -261,6 +261,22 @@ def test_row_runs_with_tiles_of_128_floats(config_guard, F):
     assert np.array_equal(_run_sddmm(coo, isrc, idst), ref.sddmm_f64(coo.row, coo.col, isrc, idst).astype(np.float32))
 
 
+@pytest.mark.parametrize("F", [64, 128, 200])
+def test_default_plan_of_a_matrix_wider_than_one_column_block(config_guard, F):
+    """40,000 columns: the library sizes the blocks itself (three of the default width, each cut in two), and
+    feature rows of 128 floats and more take 128-float tiles over passes of one block."""
+    adj = datasets.powerlaw_csr(40000, 60.0, 0.9, 2000, seed=3)
+    coo = adj.tocoo()
+    src, dst = datasets.sddmm_operands(coo, F)
+    module = VanillaSDDMMhip(coo)
+    text = _describe(module, src, dst)
+    assert "row runs" in text and ("tile=128 floats" in text) == (F >= 128), text
+    assert ("%d column blocks" % (6 if F >= 128 else 3)) in text, text
+    module.build([placeholder(src.shape), placeholder(dst.shape)], {}, {})
+    out = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
+    np.testing.assert_allclose(out, ref.sddmm_f64(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
+
+
 def test_row_runs_only_for_row_sorted_lists(config_guard):
     _lib.config_set("sddmm.blocked", 1)
     _lib.config_set("sddmm.block_cols", 500)
