@@ -123,7 +123,7 @@ def main():
     ap.add_argument("--feat-len", type=int, default=64, help="feature length of the timed step")
     ap.add_argument("--graph", default="c2", help="named synthetic configuration (featgraph_amd.datasets.CONFIGS)")
     ap.add_argument("--only", choices=["all", "spmm", "sddmm", "copy", "mh_sddmm", "mh_spmm", "mh_sddmm_softmax",
-                                       "mh_attention", "mh_attention_kv", "gather_probe"],
+                                       "mh_attention", "mh_attention_kv", "gather_probe", "gather_store_probe"],
                     default="all",
                     help="spmm / sddmm / copy / gather_probe: run just that kernel (for profiler runs), no sweep, no "
                          "CPU leg; mh_sddmm / mh_spmm: the multi-head operators (8 heads of --feat-len floats, use "
@@ -232,6 +232,17 @@ def main():
         feat_t = device_normal((n_cols, F), 1)
         p = gather_probe(feat_t, nnz, args.steps)
         print(json.dumps({"kernel": "gather_probe", "F": F, **(p or {})}))
+        return
+
+    if args.only == "gather_store_probe":
+        # whole rows of 8 x F floats from anywhere in an [N, 8, F] matrix: nnz gathers alone, then with one
+        # whole-row store per destination row beside them (the mix of multi-head SpMM and of the fused attention)
+        feat_t = device_normal((n_cols, MH_HEADS, F), 1)
+        out_t = torch.zeros((n_rows, MH_HEADS, F), dtype=torch.float32, device=dev)
+        p = rows_probe(feat_t, nnz, args.steps)
+        pw = rows_write_probe(feat_t, out_t, nnz, n_rows, p["ms"], args.steps) if p else None
+        print(json.dumps({"kernel": "gather_store_probe", "graph": args.graph, "row_floats": MH_HEADS * F,
+                          "gathers": nnz, "row_stores": n_rows, "read_only": p, "with_stores": pw}))
         return
 
     def mh_case(kind, graph_adj, D, steps, warmup, check):
