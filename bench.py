@@ -241,8 +241,22 @@ def main():
         out_t = torch.zeros((n_rows, MH_HEADS, F), dtype=torch.float32, device=dev)
         p = rows_probe(feat_t, nnz, args.steps)
         pw = rows_write_probe(feat_t, out_t, nnz, n_rows, p["ms"], args.steps) if p else None
-        print(json.dumps({"kernel": "gather_store_probe", "graph": args.graph, "row_floats": MH_HEADS * F,
-                          "gathers": nnz, "row_stores": n_rows, "read_only": p, "with_stores": pw}))
+        rf = MH_HEADS * F
+
+        def stores_only():
+            return L.fg_probe_store_rows_f32(out_t.data_ptr(), n_rows, rf, n_rows, stream.cuda_stream)
+
+        def one_after_the_other():
+            _lib.check(L.fg_probe_gather_rows_f32(feat_t.data_ptr(), n_cols, rf, nnz, sink.data_ptr(),
+                                                  stream.cuda_stream))
+            stores_only()
+
+        stored = stores_only()
+        alone = {"ms": timed(stores_only, args.steps, 1), "row_stores": stored} if stored > 0 else None
+        after = {"ms": timed(one_after_the_other, args.steps, 1)} if stored > 0 and p else None
+        print(json.dumps({"kernel": "gather_store_probe", "graph": args.graph, "row_floats": rf,
+                          "gathers": nnz, "row_stores": n_rows, "read_only": p, "with_stores": pw,
+                          "stores_only": alone, "gathers_then_stores": after}))
         return
 
     def mh_case(kind, graph_adj, D, steps, warmup, check):

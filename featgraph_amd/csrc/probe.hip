@@ -98,6 +98,23 @@ __global__ __launch_bounds__(fg::kBlockThreads) void probe_rows_kernel(const flo
   if (acc.x + acc.y + acc.z + acc.w == __builtin_inff()) sink[0] = acc.x;
 }
 
+// Stores alone: every group of LPR lanes writes `rows_each` whole rows of `out`, random ones.
+template <int LPR, int NV>
+__global__ __launch_bounds__(fg::kBlockThreads) void probe_store_rows_kernel(float *out, int64_t row_floats,
+                                                                             uint32_t out_rows, int rows_each) {
+  const int lane = threadIdx.x & (fg::kWaveSize - 1);
+  const int gl = lane & (LPR - 1), g = lane / LPR;
+  const uint32_t wave = blockIdx.x * fg::kWavesPerBlock + (threadIdx.x >> 6);
+  uint32_t s = wave * 2654435761u + static_cast<uint32_t>(g) * 40503u + 777u;
+  const float4 v = make_float4(1.0f, 2.0f, 3.0f, static_cast<float>(lane));
+  for (int it = 0; it < rows_each; ++it) {
+    s = s * 1664525u + 1013904223u;
+    float *q = out + static_cast<int64_t>((s >> 5) % out_rows) * row_floats + gl * 4;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) *reinterpret_cast<float4 *>(q + k * 256) = v;
+  }
+}
+
 // (lanes per row, loads per lane, rows per iteration of the grid) for a row length, or false.
 bool rows_shape(int32_t row_floats, int *lpr, int *nv, int64_t *per_iter) {
   if (row_floats == 128)
@@ -184,6 +201,35 @@ extern "C" int fg_probe_gather_write_rows_count(int32_t row_floats, int64_t n_ga
   *gathers = iters * per_iter;
   *writes = groups * (iters / rows_write_every(nv, gathers_per_write));
   return FG_OK;
+}
+
+extern "C" int64_t fg_probe_store_rows_f32(float *out, int64_t n_out_rows, int32_t row_floats, int64_t n_stores,
+                                           void *stream) {
+  int lpr, nv;
+  int64_t per_iter;
+  if (!out || !rows_shape(row_floats, &lpr, &nv, &per_iter) || n_out_rows < 1 || n_out_rows > 0xffffffffLL ||
+      n_stores < 0 || !fg::aligned_to(out, 16)) {
+    fg::fail(FG_EINVAL, "out, row_floats (128, 256, 512 or 1024), n_out_rows or n_stores out of range");
+    return -1;
+  }
+  const int64_t groups = int64_t{kProbeBlocks} * fg::kWavesPerBlock * (fg::kWaveSize / lpr);
+  const int rows_each = static_cast<int>(std::max<int64_t>(1, (n_stores + groups / 2) / groups));
+  const uint32_t no = static_cast<uint32_t>(n_out_rows);
+  const dim3 grid(kProbeBlocks), block(fg::kBlockThreads);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (row_floats == 128)
+    probe_store_rows_kernel<32, 1><<<grid, block, 0, st>>>(out, row_floats, no, rows_each);
+  else if (row_floats == 256)
+    probe_store_rows_kernel<64, 1><<<grid, block, 0, st>>>(out, row_floats, no, rows_each);
+  else if (row_floats == 512)
+    probe_store_rows_kernel<64, 2><<<grid, block, 0, st>>>(out, row_floats, no, rows_each);
+  else
+    probe_store_rows_kernel<64, 4><<<grid, block, 0, st>>>(out, row_floats, no, rows_each);
+  if (hipGetLastError() != hipSuccess) {
+    fg::fail(FG_EHIP, "probe launch failed");
+    return -1;
+  }
+  return groups * rows_each;  // rows stored
 }
 
 extern "C" int fg_probe_gather_f32(const float *feat, int64_t n_rows, int32_t F, int32_t tile, int32_t band_rows,

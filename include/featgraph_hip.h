@@ -317,6 +317,15 @@ FG_API int fg_probe_gather_write_rows_f32(const float *feat, int64_t n_rows, int
                                           void *stream);
 FG_API int fg_probe_gather_write_rows_count(int32_t row_floats, int64_t n_gathers, int32_t gathers_per_write,
                                             int64_t *gathers, int64_t *writes);
+/*
+ * The stores alone: about n_stores whole rows of out [n_out_rows, row_floats],
+ * random ones, and nothing read.  Returns the number of rows stored (the
+ * request rounded to whole rows per group of lanes), or -1 on a bad argument.
+ * Together with the probes above it separates what the stores cost by
+ * themselves from what they cost in between the gathers.
+ */
+FG_API int64_t fg_probe_store_rows_f32(float *out, int64_t n_out_rows, int32_t row_floats, int64_t n_stores,
+                                       void *stream);
 
 /*
  * Launch-shape overrides for tuning and tests.  The store is process-global

@@ -116,3 +116,4 @@ def test_error_codes_of_the_later_entry_points_without_a_device():
     assert g.value >= 60_000_000 and 20 <= g.value / w.value <= 30                        # about one write per 25 gathers
     assert L.fg_probe_gather_write_rows_count(100, 10, 25, ctypes.byref(g), ctypes.byref(w)) == -1
     assert L.fg_attention_csr_mh_f32(None, None, None, None, None, 8, 64, None) == -1
+    assert L.fg_probe_store_rows_f32(None, 4, 512, 10, None) == -1 and L.fg_probe_store_rows_f32(16, 4, 100, 10, None) == -1
