@@ -638,6 +638,20 @@ def main():
                           args.graph, F, sorted(per_p), best, cores, per_p[best]["runs"])}
         result["parity"] = {"spmm_bit_exact_vs_cpu_restatement": bool(np.array_equal(gpu_out, cpu_out)),
                             "spmm_max_abs_diff": float(np.max(np.abs(gpu_out - cpu_out)))}
+        # distance of the float32 result (the reference's summation order) from the exact sum, by row degree
+        exact = ref.spmm_csr_f64(adj.indptr, adj.indices, adj.data, feat_np)
+        err = np.abs(gpu_out.astype(np.float64) - exact).max(axis=1)
+        mag = np.abs(exact).max(axis=1)
+        deg = np.diff(adj.indptr)
+        bins = []
+        for lo_d, hi_d in ((0, 64), (64, 512), (512, 4096), (4096, 1 << 30)):
+            sel = (deg >= lo_d) & (deg < hi_d)
+            if sel.any():
+                bins.append({"degree": "%d..%s" % (lo_d, hi_d - 1 if hi_d < (1 << 30) else "max"),
+                             "rows": int(sel.sum()), "max_abs_err": float(err[sel].max()),
+                             "max_err_over_row_magnitude": float((err[sel] / np.maximum(mag[sel], 1e-30)).max())})
+        result["parity"]["spmm_float32_vs_exact_sum_by_row_degree"] = bins
+        del exact, err, mag
         if "sweep" in result:
             result["parity"]["every_sweep_row_passes"] = all(
                 all(v for k, v in r["parity"].items() if isinstance(v, bool)) for r in result["sweep"] if "parity" in r)
@@ -655,13 +669,27 @@ def main():
         t0 = time.time()
         ref.sddmm_x86_fast(coo.row[:m], coo.col[:m], src, dst, False, buf)
         simd_s = time.time() - t0
+        # courtesy number, not the reference's schedule: the whole edge list, edge-parallel on every core
+        full = np.empty(nnz, dtype=np.float32)
+        ref.sddmm_x86_fast(coo.row, coo.col, src, dst, True, full)
+        t0 = time.time()
+        ref.sddmm_x86_fast(coo.row, coo.col, src, dst, True, full)
+        all_cores_s = time.time() - t0
+        del full
         result["cpu_baseline_sddmm"] = {
             "value": 2.0 * m * F / strict_s / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
             "cpu_model": cpu_model(),
+            "value_all_cores_edge_parallel_not_the_reference_schedule": 2.0 * nnz * F / all_cores_s / 1e9,
+            "all_cores": cores,
             "variant": "strict serial nest: edge loop outside, k loop inside, sequential float32 sum "
                        "(op/vanilla_sddmm.py:43-47 under the default schedule :66-74, which has no parallel axis)",
             "value_with_reassociated_simd_k_loop": 2.0 * m * F / simd_s / 1e9,
             "sample": "first %d edges of the row-sorted COO list, feat-len %d, one run after one warm-up" % (m, F)}
+    try:
+        import tvm  # noqa: F401  (the reference's code generator; not expected on this machine)
+        result["tvm_available"] = True
+    except Exception:
+        result["tvm_available"] = False
     print(json.dumps(result))
 
 
