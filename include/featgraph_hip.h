@@ -360,10 +360,13 @@ FG_API int64_t fg_probe_store_rows_f32(float *out, int64_t n_out_rows, int32_t r
  * "sddmm.rows_wide" (1: 64-float tiles only, 2: 128-float tiles over passes of
  * half the width for feature rows of 128 floats and more; by default 2 when a
  * (row, pass) run then still holds 8 edges on average),
- * "attention.blocks" (grid size of the fused attention kernel).  Value 0 restores the default of
- * a size; for the 0/1 flags a negative value does.
- * The spmm.* keys change the launch shape only; "sddmm.group" also changes the
- * shape of the summation tree, i.e. the last bits of an SDDMM result.
+ * "attention.blocks" (grid size of the fused attention kernel; by default one
+ * vertex row per wave when a row is 1 KB or more, else 65536 workgroups that
+ * walk the rows).  Value 0 restores the default of a size; for the 0/1 flags a
+ * negative value does.
+ * The spmm.* keys change the launch shape only; "sddmm.group" and
+ * "sddmm.rows_wide" also change the shape of the summation tree, i.e. the last
+ * bits of an SDDMM result.
  */
 FG_API int fg_config_set(const char *key, int32_t value);
 FG_API int fg_config_get(const char *key, int32_t *value);
