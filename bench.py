@@ -139,7 +139,7 @@ def main():
     import numpy as np
     import torch
     from featgraph_amd import _lib, datasets, nd, placeholder
-    from featgraph_amd.module import (EdgeSoftmaxhip, MultiHeadAttentionhip, MultiHeadSDDMMhip,
+    from featgraph_amd.module import (EdgeSoftmaxhip, GeneralizedSpMMhip, MultiHeadAttentionhip, MultiHeadSDDMMhip,
                                       MultiHeadSDDMMSoftmaxhip, MultiHeadSpMMhip, VanillaSDDMMhip, VanillaSpMMhip)
 
     L = _lib.lib()  # fail now if the HIP library is missing
@@ -528,6 +528,28 @@ def main():
                       "frac": b / sec / 1e9 / HBM_PEAK_GBPS})
         log("sddmm on the shuffled list, F=%d: %.3f ms" % (F, sec * 1e3))
         del shuffled, ins
+        torch.cuda.empty_cache()
+
+        # the generalised aggregation (message x reducer) at the headline length: same gathers as the vanilla
+        # operator, one more operand per nonzero when the message uses the edge value
+        x = spmm_case(F)
+        for msg, reduce in (("mul", "sum"), ("copy_u", "max"), ("add", "min"), ("mul", "mean")):
+            general = GeneralizedSpMMhip(adj, msg, reduce)
+            general.build([placeholder((n_cols, F))], {}, {})
+            ramp(lambda: general.run([x]))
+            sec = general.measure_average_time([x], 5)
+            b = spmm_alg_bytes(nnz, n_rows, F)
+            row = {"op": "spmm_general", "msg": msg, "reduce": reduce, "F": F, "ms": sec * 1e3,
+                   "alg_GBps": b / sec / 1e9, "frac": b / sec / 1e9 / HBM_PEAK_GBPS}
+            if check:
+                want = ref.spmm_general(adj.indptr, adj.indices, adj.data, x.tensor.cpu().numpy(), msg, reduce)
+                row["parity"] = {"bit_exact_vs_cpu_restatement":
+                                 bool(np.array_equal(general.out_tvm.asnumpy(), want, equal_nan=True))}
+                del want
+            sweep.append(row)
+            log("spmm_general %s/%s F=%d: %.3f ms" % (msg, reduce, F, sec * 1e3))
+            del general
+        del x
         torch.cuda.empty_cache()
         result["sweep"] = sweep
 

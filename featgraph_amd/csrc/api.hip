@@ -618,9 +618,7 @@ int fg_spmm_csr_general_f32(const fg_spmm_plan *plan, const float *feat, const f
   if (plan->nnz > 0 && (!feat || (!vals && msg != FG_MSG_COPY_U)))
     return fg::fail(FG_EINVAL, "feat or edge values are null");
   if (plan->n_rows == 0) return FG_OK;
-  const int32_t *lo = plan->seg;  // whole rows, in the plan's visiting order
-  const int32_t *hi = plan->seg + static_cast<int64_t>(plan->n_blocks) * plan->n_rows;
-  return fg::spmm_general_launch(plan->row_order, lo, hi, plan->indices, vals, feat, out,
+  return fg::spmm_general_launch(plan->row_order, plan->seg, plan->n_blocks, plan->indices, vals, feat, out,
                                  static_cast<int32_t>(plan->n_rows), F, msg, reduce, static_cast<hipStream_t>(stream));
 }
 

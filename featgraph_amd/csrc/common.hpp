@@ -151,7 +151,7 @@ int sddmm_rows_launch(const int32_t *seg, const int32_t *row_order, int32_t n_ro
                       int64_t src_bytes, int64_t dst_bytes, int32_t F, hipStream_t stream);
 
 // Generalised operators (general.hip): msg / reduce / op are the FG_MSG_* / FG_REDUCE_* / FG_EDGE_* codes.
-int spmm_general_launch(const int32_t *row_order, const int32_t *seg_lo, const int32_t *seg_hi, const int32_t *indices,
+int spmm_general_launch(const int32_t *row_order, const int32_t *seg, int32_t n_blocks, const int32_t *indices,
                         const float *vals, const float *feat, float *out, int32_t n_rows, int32_t F, int msg,
                         int reduce, hipStream_t stream);
 int sddmm_elementwise_launch(const int32_t *row, const int32_t *col, const float *src, const float *dst, float *out,

@@ -30,13 +30,6 @@ __device__ __forceinline__ float message(float u, float e) {
 }
 
 template <int RED>
-__device__ __forceinline__ float fold_init() {
-  if constexpr (RED == FG_REDUCE_MAX) return -__builtin_inff();
-  if constexpr (RED == FG_REDUCE_MIN) return __builtin_inff();
-  return 0.0f;
-}
-
-template <int RED>
 __device__ __forceinline__ float fold(float acc, float t) {
   if constexpr (RED == FG_REDUCE_MAX) return (t > acc) ? t : acc;
   if constexpr (RED == FG_REDUCE_MIN) return (t < acc) ? t : acc;
@@ -45,8 +38,11 @@ __device__ __forceinline__ float fold(float acc, float t) {
 
 struct GeneralArgs {
   const int32_t *row_order;  // rows by descending degree
-  const int32_t *seg_lo;     // bounds of each row, in that order
-  const int32_t *seg_hi;
+  const int32_t *seg_lo;     // bounds, in that order, of the part of each row that this launch covers: the
+  const int32_t *seg_hi;     // whole row, or its nonzeros inside one column block (a pass)
+  const int32_t *row_lo;     // bounds of the whole rows
+  const int32_t *row_hi;
+  bool first_pass;           // the launch that writes the zeros of rows without nonzeros
   const int32_t *indices;
   const float *vals;
   const float *feat;
@@ -58,7 +54,7 @@ template <int VEC, int LPR, int MSG, int RED>
 __global__ __launch_bounds__(kBlockThreads) void spmm_general_kernel(const GeneralArgs a) {
   constexpr int RPW = kWaveSize / LPR;
   constexpr int TW = VEC * LPR;
-  constexpr int U = 8;
+  constexpr int U = 16;
   const int lane = threadIdx.x & (kWaveSize - 1);
   const int sl = lane & (LPR - 1);
   const int64_t slot = (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6)) * RPW + lane / LPR;
@@ -66,21 +62,54 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_general_kernel(const Gener
   const int tile = static_cast<int>(slot / a.n_rows);
   const int i = static_cast<int>(slot - static_cast<int64_t>(tile) * a.n_rows);
   const int row = a.row_order[i];
+  const int first = a.seg_lo[i], end = a.seg_hi[i];
+  const int row_first = a.row_lo[i], row_end = a.row_hi[i];
   const int f0 = tile * TW + sl * VEC;
   const bool fok = f0 < a.F;  // lanes past a partial last tile only serve the cross-lane reads
   const int64_t F = a.F;
   const float *fp = a.feat + (fok ? f0 : a.F - VEC);
-  const int first = a.seg_lo[i], end = a.seg_hi[i];
+  float *op = a.out + static_cast<int64_t>(row) * F + f0;
+  // A pass continues the fold where the pass before it stopped: the value it left in Out.  The pass that holds
+  // the row's first nonzero starts afresh (sum: from +0; max / min: with the first message itself, as the
+  // reference order of evaluation has it), and a pass without nonzeros of the row leaves Out alone.
+  const bool starts = first == row_first;
+  if (end <= first) {
+    if (a.first_pass && row_end <= row_first && fok) {
+      if constexpr (VEC == 4)
+        *reinterpret_cast<float4 *>(op) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      else
+        *op = 0.0f;
+    }
+    return;
+  }
   float acc[VEC];
 #pragma unroll
-  for (int k = 0; k < VEC; ++k) acc[k] = fold_init<RED>();
+  for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
+  if (!starts && fok) {
+    if constexpr (VEC == 4) {
+      const float4 q = *reinterpret_cast<const float4 *>(op);
+      acc[0] = q.x, acc[1] = q.y, acc[2] = q.z, acc[3] = q.w;
+    } else {
+      acc[0] = *op;
+    }
+  }
+  constexpr bool PICKS = RED == FG_REDUCE_MAX || RED == FG_REDUCE_MIN;
+  // ids and values of the next LPR nonzeros are requested before the gathers of the current ones
+  int next_col = 0;
+  float next_val = 1.0f;
+  if (sl < end - first) {
+    next_col = a.indices[first + sl];
+    if (MSG != FG_MSG_COPY_U) next_val = a.vals[first + sl];
+  }
   for (int e = first; e < end; e += LPR) {
     const int n = min(LPR, end - e);
-    int my_col = 0;
-    float my_val = 1.0f;
-    if (sl < n) {
-      my_col = a.indices[e + sl];
-      if (MSG != FG_MSG_COPY_U) my_val = a.vals[e + sl];
+    const int my_col = next_col;
+    const float my_val = next_val;
+    next_col = 0;
+    next_val = 1.0f;
+    if (sl < end - (e + LPR)) {
+      next_col = a.indices[e + LPR + sl];
+      if (MSG != FG_MSG_COPY_U) next_val = a.vals[e + LPR + sl];
     }
     for (int j = 0; j < n; j += U) {
       float x[U][VEC];
@@ -101,19 +130,21 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_general_kernel(const Gener
 #pragma unroll
       for (int u = 0; u < U; ++u)
         if (j + u < n) {
+          const bool very_first = PICKS && u == 0 && starts && e == first && j == 0;
 #pragma unroll
-          for (int k = 0; k < VEC; ++k) acc[k] = fold<RED>(acc[k], message<MSG>(x[u][k], v[u]));
+          for (int k = 0; k < VEC; ++k) {
+            const float t = message<MSG>(x[u][k], v[u]);
+            acc[k] = very_first ? t : fold<RED>(acc[k], t);
+          }
         }
     }
   }
   if (!fok) return;
-  const float count = static_cast<float>(end - first);
+  if (RED == FG_REDUCE_MEAN && end == row_end) {
+    const float count = static_cast<float>(row_end - row_first);
 #pragma unroll
-  for (int k = 0; k < VEC; ++k) {
-    if (end <= first) acc[k] = 0.0f;
-    else if (RED == FG_REDUCE_MEAN) acc[k] = acc[k] / count;
+    for (int k = 0; k < VEC; ++k) acc[k] = acc[k] / count;
   }
-  float *op = a.out + static_cast<int64_t>(row) * F + f0;
   if constexpr (VEC == 4)
     *reinterpret_cast<float4 *>(op) = make_float4(acc[0], acc[1], acc[2], acc[3]);
   else
@@ -203,22 +234,7 @@ int launch_elementwise(const int32_t *row, const int32_t *col, const float *src,
 
 }  // namespace
 
-int spmm_general_launch(const int32_t *row_order, const int32_t *seg_lo, const int32_t *seg_hi, const int32_t *indices,
-                        const float *vals, const float *feat, float *out, int32_t n_rows, int32_t F, int msg,
-                        int reduce, hipStream_t stream) {
-  if (n_rows == 0) return FG_OK;
-  GeneralArgs a;
-  a.row_order = row_order;
-  a.seg_lo = seg_lo;
-  a.seg_hi = seg_hi;
-  a.indices = indices;
-  a.vals = vals;
-  a.feat = feat;
-  a.out = out;
-  a.n_rows = n_rows;
-  a.F = F;
-  a.n_tiles = 1;
-  const bool vec4 = F % 4 == 0 && aligned_to(feat, 16) && aligned_to(out, 16);
+static int general_pass(GeneralArgs a, bool vec4, int msg, int reduce, hipStream_t stream) {
   switch (msg) {
     case FG_MSG_MUL: return dispatch_reduce<FG_MSG_MUL>(a, vec4, reduce, stream);
     case FG_MSG_ADD: return dispatch_reduce<FG_MSG_ADD>(a, vec4, reduce, stream);
@@ -227,6 +243,36 @@ int spmm_general_launch(const int32_t *row_order, const int32_t *seg_lo, const i
     case FG_MSG_COPY_U: return dispatch_reduce<FG_MSG_COPY_U>(a, vec4, reduce, stream);
   }
   return fail(FG_EINVAL, "msg = %d is not one of FG_MSG_MUL / ADD / SUB / DIV / COPY_U", msg);
+}
+
+// seg: the plan's bounds table, (n_blocks + 1) * n_rows entries in visiting order.  With column blocks the rows
+// are folded pass by pass in ascending column order, one launch per pass over all feature tiles, the partial
+// results carried in `out` (launches on one stream are ordered, so every element still sees its terms in CSR
+// order): the gathers of a pass then come from a band of the feature matrix that fits one L2.
+int spmm_general_launch(const int32_t *row_order, const int32_t *seg, int32_t n_blocks, const int32_t *indices,
+                        const float *vals, const float *feat, float *out, int32_t n_rows, int32_t F, int msg,
+                        int reduce, hipStream_t stream) {
+  if (n_rows == 0) return FG_OK;
+  GeneralArgs a;
+  a.row_order = row_order;
+  a.row_lo = seg;
+  a.row_hi = seg + static_cast<int64_t>(n_blocks) * n_rows;
+  a.indices = indices;
+  a.vals = vals;
+  a.feat = feat;
+  a.out = out;
+  a.n_rows = n_rows;
+  a.F = F;
+  a.n_tiles = 1;
+  const bool vec4 = F % 4 == 0 && aligned_to(feat, 16) && aligned_to(out, 16);
+  const int passes = config().spmm_blocked == 0 ? 1 : std::max(1, n_blocks);
+  for (int b = 0; b < passes; ++b) {
+    a.seg_lo = passes == 1 ? a.row_lo : seg + static_cast<int64_t>(b) * n_rows;
+    a.seg_hi = passes == 1 ? a.row_hi : seg + static_cast<int64_t>(b + 1) * n_rows;
+    a.first_pass = b == 0;
+    if (int rc = general_pass(a, vec4, msg, reduce, stream)) return rc;
+  }
+  return FG_OK;
 }
 
 int sddmm_elementwise_launch(const int32_t *row, const int32_t *col, const float *src, const float *dst, float *out,

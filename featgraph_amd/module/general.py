@@ -5,6 +5,8 @@ The reference builds its operators around two slots, a message function folded b
 each (multiply + sum, dot product) under the name "generalized SpMM / SDDMM" (README.md:6).  The classes
 here fill the slots with the other operators; the call surface is that of the vanilla modules.
 """
+import re
+
 import torch
 
 from .. import _lib
@@ -39,9 +41,14 @@ class GeneralizedSpMMhip(SpMMbase):
 
     def lower_to_ir(self, input_placeholders, compute_args, schedule_args):
         _, H, D, _ = self._parse_build(input_placeholders, compute_args, schedule_args)
-        return ("spmm_csr_general rows=%d cols=%d nnz=%d D=%d | msg=%s reduce=%s | kernel=row-slot, whole rows, "
-                "rows=by-descending-degree, tile=64 floats x %d tiles, 1 launch" % (
-                    self._num_rows, self._num_cols, self._nnz, D, self._msg, self._reduce, (D + 63) // 64))
+        # the plan's own description tells whether (and into how many) column blocks the matrix is cut
+        plan_text = super().lower_to_ir(input_placeholders, compute_args, schedule_args)
+        found = re.search(r"(\d+) column blocks of (\d+)", plan_text)
+        passes = ("%s column blocks of %s, one launch per block, the fold carried in the output" % found.groups()
+                  if found else "whole rows, 1 launch")
+        return ("spmm_csr_general rows=%d cols=%d nnz=%d D=%d | msg=%s reduce=%s | kernel=row-slot, %s, "
+                "rows=by-descending-degree, tile=64 floats x %d tiles" % (
+                    self._num_rows, self._num_cols, self._nnz, D, self._msg, self._reduce, passes, (D + 63) // 64))
 
     def _launch(self, tensors):
         feat = tensors[0]

@@ -130,8 +130,10 @@ FG_API int fg_spmm_csr_noalloc_f32(int64_t n_rows, int64_t n_cols, int64_t nnz, 
  * MEAN is the sum divided by the row's degree (one rounded division).  Rows
  * without nonzeros give 0 under every reducer.  One rounded operation per
  * message and per fold step, so (MUL, SUM) equals fg_spmm_csr_f32 bit for bit.
- * vals may be null for FG_MSG_COPY_U.  Single launch over whole rows in the
- * plan's row order.
+ * vals may be null for FG_MSG_COPY_U.  One launch per column block of the
+ * plan (one launch over whole rows when the plan has no blocks); the partial
+ * fold of a row is carried in `out` between launches, so `out` must not be
+ * read by anything else on the stream until the last launch has finished.
  */
 #define FG_MSG_MUL 0
 #define FG_MSG_ADD 1

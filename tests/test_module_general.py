@@ -56,6 +56,39 @@ def test_hub_rows_empty_rows_and_unsorted_duplicate_columns(reduce):
     assert np.all(out[[1, 3]] == 0)
 
 
+@pytest.mark.parametrize("msg", MSGS)
+@pytest.mark.parametrize("reduce", REDUCES)
+def test_column_block_passes_fold_in_the_same_order(msg, reduce):
+    """With column blocks the fold of a row runs pass by pass, its state carried in the output: the same bits as
+    the single pass, for blocks so narrow that many (row, pass) runs are empty and rows start in a late pass, with
+    rows without nonzeros, and with a not-a-number as a row's first and as a later message."""
+    from featgraph_amd import _lib
+    adj = datasets.config_graph("c2-mini").tolil()
+    adj[5] = 0
+    adj[4242] = 0
+    adj = adj.tocsr()
+    adj.sort_indices()
+    adj.data = (adj.data + np.float32(0.25)).astype(np.float32)
+    feat = datasets.spmm_operands(adj, 72)                # a whole tile and a partial one
+    feat[adj.indices[adj.indptr[7]]] = np.nan             # first message of row 7 (and wherever else the vertex occurs)
+    feat[adj.indices[adj.indptr[9] + 3]] = np.nan         # a later message of row 9
+    want = ref.spmm_general(adj.indptr, adj.indices, adj.data, feat, msg, reduce)
+    try:
+        _lib.config_set("spmm.blocked", 1)
+        for block_cols in (64, 1500):
+            _lib.config_set("spmm.block_cols", block_cols)
+            module = GeneralizedSpMMhip(adj, msg, reduce)
+            assert "column blocks" in module.lower_to_ir([placeholder(feat.shape)], {}, {})
+            module.build([placeholder(feat.shape)], {}, {})
+            module.out_tvm.tensor.fill_(7.0)
+            out = module.run([nd.array(feat, module.ctx)]).asnumpy()
+            assert np.array_equal(out, want, equal_nan=True), block_cols
+            assert not out[5].any() and not out[4242].any()
+    finally:
+        _lib.config_set("spmm.blocked", -1)
+        _lib.config_set("spmm.block_cols", 0)
+
+
 def test_mul_sum_is_the_vanilla_kernel_and_max_min_match_numpy(adj_127x255):
     adj = adj_127x255
     feat = np.random.default_rng(2).standard_normal((adj.shape[1], 96), dtype=np.float32)
