@@ -513,21 +513,29 @@ def main():
                 f, sweep[-2]["ms"], sweep[-2]["frac_of_gather_ceiling"] or 0, sweep[-1]["ms"],
                 sweep[-1]["frac_of_gather_ceiling"] or 0))
 
-        # the same edge list in a seeded random order: not row-sorted, so the re-ordered edge-list kernels run
+        # the same edge list in a seeded random order: not row-sorted, so the plan works on a sorted copy and
+        # gathers the results back to the caller's order
         import scipy.sparse
         perm = np.random.default_rng(17).permutation(nnz)
         shuffled = VanillaSDDMMhip(scipy.sparse.coo_matrix((coo.data[perm], (coo.row[perm], coo.col[perm])),
                                                            shape=coo.shape))
-        del perm
         ins = sddmm_case(shuffled, F)
         ramp(lambda: shuffled.run(ins))
         sec = shuffled.measure_average_time(ins, 5)
         b = sddmm_alg_bytes(nnz, F)
-        sweep.append({"op": "sddmm", "F": F, "edge_order": "shuffled (seeded permutation of the c2 list)",
-                      "ms": sec * 1e3, "GFLOPs": 2.0 * nnz * F / sec / 1e9, "alg_GBps": b / sec / 1e9,
-                      "frac": b / sec / 1e9 / HBM_PEAK_GBPS})
+        row = {"op": "sddmm", "F": F, "edge_order": "shuffled (seeded permutation of the c2 list)",
+               "ms": sec * 1e3, "GFLOPs": 2.0 * nnz * F / sec / 1e9, "alg_GBps": b / sec / 1e9,
+               "frac": b / sec / 1e9 / HBM_PEAK_GBPS}
+        if check:
+            out = shuffled.out_tvm.asnumpy()[:m]
+            exact = ref.sddmm_f64(coo.row[perm[:m]], coo.col[perm[:m]], ins[0].tensor.cpu().numpy(),
+                                  ins[1].tensor.cpu().numpy())
+            row["parity"] = {"within_rtol1e-5_atol1e-4_of_float64":
+                             bool(np.all(np.abs(out - exact) <= ATOL + RTOL * np.abs(exact))), "edges_checked": m}
+            del out, exact
+        sweep.append(row)
         log("sddmm on the shuffled list, F=%d: %.3f ms" % (F, sec * 1e3))
-        del shuffled, ins
+        del shuffled, ins, perm
         torch.cuda.empty_cache()
 
         # the generalised aggregation (message x reducer) at the headline length: same gathers as the vanilla

@@ -75,6 +75,9 @@ struct fg_sddmm_plan {
   // it (visiting order + per-column-block bounds) for the row-run kernel.  Null otherwise.
   int32_t *indptr = nullptr;      // owned, device, n_rows + 1 entries
   fg_spmm_plan *rows = nullptr;   // owned
+  // Any other list with valid ids: a copy sorted by (row, column), over which `indptr` and `rows` are then
+  // built; the row-run kernel writes its results in that order and a gather returns them to the caller's.
+  fg::SddmmSorted sorted;
 };
 
 static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr, const int32_t *indices,
@@ -431,6 +434,7 @@ int *config_slot(const char *key) {
   if (!strcmp(key, "sddmm.rows")) return &c.sddmm_rows;
   if (!strcmp(key, "sddmm.rows_blocks")) return &c.sddmm_rows_blocks;
   if (!strcmp(key, "sddmm.rows_wide")) return &c.sddmm_rows_wide;
+  if (!strcmp(key, "sddmm.sorted_copy")) return &c.sddmm_sorted_copy;
   if (!strcmp(key, "attention.blocks")) return &c.attention_blocks;
   return nullptr;
 }
@@ -663,20 +667,42 @@ static int build_row_runs(fg_sddmm_plan *p, int32_t num_col_partitions) {
   if (err == hipSuccess) err = hipMemcpy(&bad, flag, sizeof(int), hipMemcpyDeviceToHost);
   (void)hipFree(flag);
   if (err != hipSuccess) return fg::fail(FG_EHIP, "row order check: %s", hipGetErrorString(err));
-  if (bad) return FG_OK;
+  const int32_t *rows_of = p->row, *cols_of = p->col;
+  if (bad) {
+    // not row-sorted (or ids outside the matrix, which the sort refuses): work on a sorted copy
+    if (fg::config().sddmm_sorted_copy == 0 || fg::config().sddmm_blocked == 0) return FG_OK;
+    if (int rc = fg::sddmm_sorted_build(p->nnz, p->n_rows, p->n_cols, p->row, p->col, &p->sorted)) return rc;
+    if (!p->sorted.col_s) return FG_OK;
+    rows_of = p->sorted.row_s;
+    cols_of = p->sorted.col_s;
+  }
   err = hipMalloc(&p->indptr, sizeof(int32_t) * (p->n_rows + 1));
   if (err != hipSuccess) {
     p->indptr = nullptr;
     return fg::fail(err == hipErrorOutOfMemory ? FG_ENOMEM : FG_EHIP, "row pointer: %s", hipGetErrorString(err));
   }
-  indptr_from_rows_kernel<<<dim3(grid), dim3(256)>>>(p->row, p->nnz, static_cast<int32_t>(p->n_rows), p->indptr);
+  indptr_from_rows_kernel<<<dim3(grid), dim3(256)>>>(rows_of, p->nnz, static_cast<int32_t>(p->n_rows), p->indptr);
   FG_HIP_TRY(hipGetLastError());
   FG_HIP_TRY(hipDeviceSynchronize());
+  if (p->sorted.row_s) {
+    (void)hipFree(p->sorted.row_s);
+    p->sorted.row_s = nullptr;
+  }
   // same block width as the re-ordered edge list (sddmm_blocked.hip); a run costs a wave a fixed amount of
   // work, so blocks need 8 edges per run on average (sparser lists keep whole rows and take the edge-list path)
-  return row_plan_create(p->n_rows, p->n_cols, p->nnz, p->indptr, p->col, num_col_partitions,
-                         fg::config().sddmm_block_cols, kSddmmBlockCols, kSddmmSplit, fg::config().sddmm_blocked, 8.0,
-                         false, &p->rows);
+  if (int rc = row_plan_create(p->n_rows, p->n_cols, p->nnz, p->indptr, cols_of, num_col_partitions,
+                               fg::config().sddmm_block_cols, kSddmmBlockCols, kSddmmSplit, fg::config().sddmm_blocked,
+                               8.0, false, &p->rows))
+    return rc;
+  if (p->sorted.col_s && !(p->rows && p->rows->seg && p->rows->n_blocks >= 2)) {
+    // too thin for column blocks: the sorted copy would buy nothing over the caller's list
+    if (p->rows) fg_spmm_plan_destroy(p->rows);
+    p->rows = nullptr;
+    (void)hipFree(p->indptr);
+    p->indptr = nullptr;
+    fg::sddmm_sorted_free(&p->sorted);
+  }
+  return FG_OK;
 }
 
 int fg_sddmm_plan_create(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,
@@ -726,6 +752,7 @@ int fg_sddmm_plan_create_partitioned(int64_t nnz, int64_t n_rows, int64_t n_cols
 void fg_sddmm_plan_destroy(fg_sddmm_plan *plan) {
   if (!plan) return;
   fg::sddmm_blocks_free(&plan->blocks);
+  fg::sddmm_sorted_free(&plan->sorted);
   if (plan->rows) fg_spmm_plan_destroy(plan->rows);
   if (plan->indptr) (void)hipFree(plan->indptr);
   delete plan;
@@ -780,10 +807,14 @@ int fg_sddmm_coo_plan_f32(const fg_sddmm_plan *plan, const float *src, const flo
     if (int rc = check_heads(H, D)) return rc;
     if (!src || !dst || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
     const fg_spmm_plan *r = plan->rows;
-    return fg::sddmm_rows_launch(r->seg, r->row_order, static_cast<int32_t>(r->n_rows), r->n_blocks,
-                                 sddmm_rows_merge64(plan), sddmm_rows_max_wide(plan), plan->col, src,
-                                 dst, out, plan->n_cols * int64_t{D} * 4, plan->n_rows * int64_t{D} * 4, D,
-                                 static_cast<hipStream_t>(stream));
+    const bool copy = plan->sorted.col_s != nullptr;
+    if (int rc = fg::sddmm_rows_launch(r->seg, r->row_order, static_cast<int32_t>(r->n_rows), r->n_blocks,
+                                       sddmm_rows_merge64(plan), sddmm_rows_max_wide(plan),
+                                       copy ? plan->sorted.col_s : plan->col, src, dst,
+                                       copy ? plan->sorted.results : out, plan->n_cols * int64_t{D} * 4,
+                                       plan->n_rows * int64_t{D} * 4, D, static_cast<hipStream_t>(stream)))
+      return rc;
+    return copy ? fg::sddmm_unsort_launch(plan->sorted, plan->nnz, out, static_cast<hipStream_t>(stream)) : FG_OK;
   }
   if (!sddmm_use_blocks(plan, src, dst, H, D)) {
     fg::SddmmArgs a;
@@ -814,7 +845,7 @@ int fg_sddmm_softmax_plan_f32(const fg_sddmm_plan *plan, const float *src, const
   if (plan->nnz == 0) return FG_OK;
   if (int rc = check_device(plan->device)) return rc;
   if (!src || !dst || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
-  if (!plan->indptr || !plan->rows)
+  if (!plan->indptr || !plan->rows || plan->sorted.col_s)
     return fg::fail(FG_EUNSUPPORTED, "edge softmax needs a row-sorted edge list (each destination row's edges consecutive)");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int32_t n = static_cast<int32_t>(plan->n_rows);
@@ -851,10 +882,13 @@ int fg_sddmm_plan_describe(const fg_sddmm_plan *plan, int32_t H, int32_t D, char
     const int merge64 = sddmm_rows_merge64(plan);
     const int merge = merge64 == 0 ? 1 : rows_tile <= 64 ? merge64 * (64 / rows_tile) : std::max(1, merge64 / (rows_tile / 64));
     snprintf(buf, static_cast<size_t>(cap),
-             "sddmm_coo nnz=%lld H=%d D=%d | kernel=row runs (row-sorted edge list), %d column blocks of %d, tile=%d "
+             "sddmm_coo nnz=%lld H=%d D=%d | kernel=row runs (%s), %d column blocks of %d, tile=%d "
              "floats x %d tiles (one launch each), floats/lane=%d lanes/dot=%d | grid=(blocks, column blocks) x %d "
              "threads each",
-             (long long)plan->nnz, H, D, (plan->rows->n_blocks + merge - 1) / merge,
+             (long long)plan->nnz, H, D,
+             plan->sorted.col_s ? "copy of the edge list sorted by row and column, results gathered back to the caller's order"
+                                : "row-sorted edge list",
+             (plan->rows->n_blocks + merge - 1) / merge,
              static_cast<int>(std::min<int64_t>(int64_t{plan->rows->block_cols} * merge, 0x7fffffff)), rows_tile,
              (D + rows_tile - 1) / rows_tile, rows_tile <= 64 ? 4 : rows_tile / 16, std::min(rows_tile / 4, 16),
              fg::kBlockThreads);
@@ -901,7 +935,7 @@ int fg_config_set(const char *key, int32_t value) {
                     slot == &fg::config().sddmm_blocked ||
                     slot == &fg::config().spmm_buffer_loads || slot == &fg::config().sddmm_fast ||
                     slot == &fg::config().sddmm_buffer_loads || slot == &fg::config().sddmm_rows ||
-                    slot == &fg::config().spmm_multi;
+                    slot == &fg::config().spmm_multi || slot == &fg::config().sddmm_sorted_copy;
   // flags: 0 / 1 are explicit, anything negative restores the default;
   // sizes: 0 restores the default
   *slot = flag ? (value < 0 ? -1 : (value != 0)) : std::max(value, 0);

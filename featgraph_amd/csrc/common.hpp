@@ -28,7 +28,7 @@ struct Config {
   int spmm_multi = -1, spmm_multi_blocks = 0, spmm_multi_long = 0, spmm_tile_interleave = 0;
   int sddmm_group = 0, sddmm_batches = 0, sddmm_blocked = -1, sddmm_block_cols = 0;
   int sddmm_fast = -1, sddmm_buffer_loads = -1, sddmm_rows = -1, sddmm_rows_blocks = 0;
-  int attention_blocks = 0, sddmm_rows_wide = 0;
+  int attention_blocks = 0, sddmm_rows_wide = 0, sddmm_sorted_copy = -1;
 };
 Config &config();
 
@@ -125,6 +125,21 @@ struct SddmmBlocks {
   int32_t n_blocks = 0;
   int32_t block_cols = 0;
 };
+
+// Copy of a COO edge list sorted by (row, column) (sddmm_blocked.hip): lets the row-run kernel serve a list in
+// any order.  Device arrays owned by the SDDMM plan, all null when there is no such copy.
+struct SddmmSorted {
+  int32_t *row_s = nullptr;    // [nnz] row ids in sorted order; freed once the row pointer is built
+  int32_t *col_s = nullptr;    // [nnz] column ids in sorted order
+  int32_t *where = nullptr;    // [nnz] place of the caller's edge e in the sorted list
+  float *results = nullptr;    // [nnz] the dot products in sorted order, between the kernel and the gather back
+};
+// Leaves *out empty (and returns FG_OK) for ids outside the matrix, sizes beyond int32 or when memory runs out.
+int sddmm_sorted_build(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,
+                       SddmmSorted *out);
+void sddmm_sorted_free(SddmmSorted *s);
+// out[e] = s.results[s.where[e]]
+int sddmm_unsort_launch(const SddmmSorted &s, int64_t nnz, float *out, hipStream_t stream);
 
 // num_col_partitions: 0 lets the library decide, 1 builds nothing, P > 1 builds P column blocks.
 int sddmm_blocks_build(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,

@@ -12,7 +12,10 @@
 //
 // SpMM kernel: rows come in the plan's order (descending degree); a slot of LPR lanes owns one (row, tile)
 // pair, every lane VEC adjacent floats; column ids and values are fetched LPR at a time with one coalesced
-// load and handed out inside the slot with cross-lane reads; eight gathers are in flight per lane.
+// load, a chunk ahead of their use, and handed out inside the slot with cross-lane reads; sixteen gathers are
+// in flight per lane.  When the plan has column blocks the operator is one launch per block, each over the
+// block's part of every row with the partial fold carried in Out, so a launch gathers from a band of the
+// feature matrix that an L2 holds.
 #include <algorithm>
 
 #include "common.hpp"

@@ -52,7 +52,128 @@ __global__ void gather_edges_kernel(const int32_t *row, const int32_t *col, cons
   }
 }
 
+// Sort key of an edge for the (row, column) order: row id above the column id.  Raises *bad for ids outside the
+// matrix (such a list is left to the kernels that check nothing but gather nothing out of range either).
+__global__ void row_col_keys_kernel(const int32_t *row, const int32_t *col, int64_t nnz, int32_t n_rows,
+                                    int32_t n_cols, int col_bits, uint64_t *keys, int32_t *ids, int *bad) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  int b = 0;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
+    const int32_t r = row[i], c = col[i];
+    b |= (r < 0 || r >= n_rows || c < 0 || c >= n_cols) ? 1 : 0;
+    keys[i] = (static_cast<uint64_t>(static_cast<uint32_t>(r)) << col_bits) | static_cast<uint32_t>(c);
+    ids[i] = static_cast<int32_t>(i);
+  }
+  if (b) atomicOr(bad, 1);
+}
+
+// Splits the sorted keys back into ids and inverts the permutation: where[e] is the place of the caller's edge e
+// in the sorted list.
+__global__ void sorted_edges_kernel(const uint64_t *keys_sorted, const int32_t *pos, int64_t nnz, int col_bits,
+                                    int32_t *row_s, int32_t *col_s, int32_t *where) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  const uint64_t mask = (uint64_t{1} << col_bits) - 1;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
+    const uint64_t k = keys_sorted[i];
+    row_s[i] = static_cast<int32_t>(k >> col_bits);
+    col_s[i] = static_cast<int32_t>(k & mask);
+    where[pos[i]] = static_cast<int32_t>(i);
+  }
+}
+
+// out[e] = sorted[where[e]]: four edges per thread, stores coalesced, loads wherever the sort put the edges.
+__global__ __launch_bounds__(256) void unsort_kernel(const float *sorted, const int32_t *where, float *out, int64_t nnz) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x * 4;
+  for (int64_t i = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4; i < nnz; i += stride) {
+    if (i + 3 < nnz && (reinterpret_cast<uintptr_t>(out + i) & 15) == 0) {
+      const int4 w = *reinterpret_cast<const int4 *>(where + i);
+      *reinterpret_cast<float4 *>(out + i) = make_float4(sorted[w.x], sorted[w.y], sorted[w.z], sorted[w.w]);
+    } else {
+      for (int64_t k = i; k < min(i + 4, nnz); ++k) out[k] = sorted[where[k]];
+    }
+  }
+}
+
 }  // namespace
+
+void sddmm_sorted_free(SddmmSorted *s) {
+  if (s->row_s) (void)hipFree(s->row_s);
+  if (s->col_s) (void)hipFree(s->col_s);
+  if (s->where) (void)hipFree(s->where);
+  if (s->results) (void)hipFree(s->results);
+  *s = SddmmSorted();
+}
+
+int sddmm_sorted_build(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,
+                       SddmmSorted *out) {
+  *out = SddmmSorted();
+  if (nnz == 0 || n_rows == 0 || n_cols == 0 || nnz > 0x7fffffffLL || n_rows >= 0x7fffffffLL || n_cols >= 0x7fffffffLL)
+    return FG_OK;
+  int col_bits = 1, row_bits = 1;
+  while ((int64_t{1} << col_bits) < n_cols) ++col_bits;
+  while ((int64_t{1} << row_bits) < n_rows) ++row_bits;
+
+  uint64_t *keys = nullptr, *keys_sorted = nullptr;
+  int32_t *ids = nullptr, *pos = nullptr;
+  int *flag = nullptr;
+  void *tmp = nullptr;
+  size_t tmp_bytes = 0;
+  int bad = 0;
+  const size_t n = static_cast<size_t>(nnz);
+  const int grid = static_cast<int>(std::min<int64_t>((nnz + 255) / 256, 65536));
+  hipError_t err = hipMalloc(&keys, n * sizeof(uint64_t));
+  if (err == hipSuccess) err = hipMalloc(&keys_sorted, n * sizeof(uint64_t));
+  if (err == hipSuccess) err = hipMalloc(&ids, n * sizeof(int32_t));
+  if (err == hipSuccess) err = hipMalloc(&pos, n * sizeof(int32_t));
+  if (err == hipSuccess) err = hipMalloc(&flag, sizeof(int));
+  if (err == hipSuccess) err = hipMalloc(&out->row_s, n * sizeof(int32_t));
+  if (err == hipSuccess) err = hipMalloc(&out->col_s, n * sizeof(int32_t));
+  if (err == hipSuccess) err = hipMalloc(&out->where, n * sizeof(int32_t));
+  if (err == hipSuccess) err = hipMalloc(&out->results, n * sizeof(float));
+  if (err == hipSuccess) err = hipMemset(flag, 0, sizeof(int));
+  if (err == hipSuccess) {
+    row_col_keys_kernel<<<dim3(grid), dim3(256)>>>(row, col, nnz, static_cast<int32_t>(n_rows),
+                                                   static_cast<int32_t>(n_cols), col_bits, keys, ids, flag);
+    err = hipGetLastError();
+  }
+  if (err == hipSuccess) err = hipMemcpy(&bad, flag, sizeof(int), hipMemcpyDeviceToHost);
+  if (err == hipSuccess && !bad)
+    err = hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, keys, keys_sorted, ids, pos, static_cast<int>(nnz), 0,
+                                             row_bits + col_bits, nullptr);
+  if (err == hipSuccess && !bad) err = hipMalloc(&tmp, tmp_bytes ? tmp_bytes : 1);
+  if (err == hipSuccess && !bad)  // stable: edges listed twice keep the caller's order
+    err = hipcub::DeviceRadixSort::SortPairs(tmp, tmp_bytes, keys, keys_sorted, ids, pos, static_cast<int>(nnz), 0,
+                                             row_bits + col_bits, nullptr);
+  if (err == hipSuccess && !bad) {
+    sorted_edges_kernel<<<dim3(grid), dim3(256)>>>(keys_sorted, pos, nnz, col_bits, out->row_s, out->col_s, out->where);
+    err = hipGetLastError();
+  }
+  if (err == hipSuccess) err = hipDeviceSynchronize();
+  if (keys) (void)hipFree(keys);
+  if (keys_sorted) (void)hipFree(keys_sorted);
+  if (ids) (void)hipFree(ids);
+  if (pos) (void)hipFree(pos);
+  if (flag) (void)hipFree(flag);
+  if (tmp) (void)hipFree(tmp);
+  if (err != hipSuccess || bad) {
+    sddmm_sorted_free(out);
+    if (err == hipSuccess) return FG_OK;
+    if (err == hipErrorOutOfMemory) {  // no room for the sorted copy: the other kernels still work
+      (void)hipGetLastError();
+      return FG_OK;
+    }
+    return fail(FG_EHIP, "SDDMM sorted edge list construction: %s", hipGetErrorString(err));
+  }
+  return FG_OK;
+}
+
+int sddmm_unsort_launch(const SddmmSorted &s, int64_t nnz, float *out, hipStream_t stream) {
+  if (nnz == 0) return FG_OK;
+  const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((nnz + 1023) / 1024, 1 << 20));
+  unsort_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(s.results, s.where, out, nnz);
+  FG_HIP_TRY(hipGetLastError());
+  return FG_OK;
+}
 
 void sddmm_blocks_free(SddmmBlocks *b) {
   if (b->row_p) (void)hipFree(b->row_p);

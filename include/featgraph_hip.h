@@ -186,13 +186,21 @@ FG_API int fg_sddmm_coo_general_f32(int64_t nnz, const int32_t *row, const int32
  * SDDMMbase.__init__ gives to 2-D graph partitioning (module/sddmm.py:45-49).
  * When the matrix is wide and dense enough: for a list whose row ids ascend
  * and whose column ids ascend inside every row (COO derived from CSR) it
- * rebuilds the row pointer and stores where every block of 16384 columns
- * starts inside every row ((n_cols/16384 + 3) * n_rows int32); for any other
- * list it stores the edge list re-ordered by blocks of 16384 columns and, inside
- * a block, by destination row (stable otherwise) together with every edge's
- * original position: 12 bytes per edge, one device radix sort.  Results are always written in the
- * caller's edge order; there is no edge_mapping to apply.  The plan BORROWS row
- * and col, which must stay alive and unchanged until fg_sddmm_plan_destroy.
+ * rebuilds the row pointer and stores where every block of columns starts
+ * inside every row ((2 * n_cols/16384 + 3) * n_rows int32).  For a list in any
+ * other order it sorts a copy of the list by (row, column) (one device radix
+ * sort, stable), builds the same tables over the copy, and keeps the copy's
+ * column ids, every edge's place in the copy and room for the results in that
+ * order: 12 bytes per edge.  A call then runs the same kernel as for a sorted
+ * list and gathers the results back, so they are always written in the
+ * caller's edge order (there is no edge_mapping to apply) and equal the sorted
+ * list's bit for bit.  Because the results pass through memory that the plan
+ * owns, two calls on ONE plan of an unsorted list must not overlap in time.
+ * Rows that ascend while their columns do not, lists with ids outside the
+ * matrix and "sddmm.sorted_copy" = 0 fall back to a copy re-ordered by column
+ * block and destination row whose kernel scatters its results.
+ * The plan BORROWS row and col, which must stay alive and unchanged until
+ * fg_sddmm_plan_destroy.
  */
 typedef struct fg_sddmm_plan fg_sddmm_plan;
 FG_API int fg_sddmm_plan_create(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,
@@ -362,6 +370,8 @@ FG_API int64_t fg_probe_store_rows_f32(float *out, int64_t n_out_rows, int32_t r
  * "sddmm.rows_wide" (1: 64-float tiles only, 2: 128-float tiles over passes of
  * half the width for feature rows of 128 floats and more; by default 2 when a
  * (row, pass) run then still holds 8 edges on average),
+ * "sddmm.sorted_copy" (0/1: whether a plan over a list that is not row-sorted
+ * works on a sorted copy, read at plan creation; default 1),
  * "attention.blocks" (grid size of the fused attention kernel; by default one
  * vertex row per wave when a row is 1 KB or more, else 65536 workgroups that
  * walk the rows).  Value 0 restores the default of a size; for the 0/1 flags a

@@ -172,28 +172,29 @@ def test_c3_sddmm_at_every_swept_feature_length(c3_sddmm_module, F):
         assert np.all(np.abs(out[sl] - serial) <= ATOL + RTOL * np.abs(serial) + slack)
 
 
-def test_c3_sddmm_on_a_shuffled_edge_list(c2):
-    """The same edges in a seeded random order: not row-sorted, so the plan re-orders the list by column block and
-    the edge-list kernels run; results must land at the caller's positions."""
+@pytest.mark.parametrize("F", [64, 256])
+def test_c3_sddmm_on_a_shuffled_edge_list(c2, F):
+    """The same edges in a seeded random order: not row-sorted, so the plan sorts a copy, the row-run kernel works
+    on the copy and a gather brings the results back; they must land at the caller's positions."""
     import scipy.sparse
     coo = c2.tocoo()
-    n, F = coo.shape[0], 64
+    n = coo.shape[0]
     perm = np.random.default_rng(17).permutation(coo.nnz)
     shuffled = scipy.sparse.coo_matrix((coo.data[perm], (coo.row[perm], coo.col[perm])), shape=coo.shape)
     module = VanillaSDDMMhip(shuffled)
     ph = [placeholder((n, F)), placeholder((n, F))]
     text = module.lower_to_ir(ph, {}, {})
-    _say("SDDMM c3 F=64, shuffled list: %s" % text)
-    assert "row runs" not in text
+    _say("SDDMM c3 F=%d, shuffled list: %s" % (F, text))
+    assert "sorted by row and column" in text
     module.build(ph, {}, {})
     src, dst = datasets.sddmm_operands(coo, F)
     out = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
     np.testing.assert_allclose(out, ref.sddmm_f64(shuffled.row, shuffled.col, src, dst), rtol=RTOL, atol=ATOL)
-    # against the sorted list's results, edge by edge: same dot products, possibly another summation tree
+    # against the sorted list's results, edge by edge: the same kernel over the same runs, so the same bits
     sorted_module = VanillaSDDMMhip(coo)
     sorted_module.build(ph, {}, {})
     base = sorted_module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
-    np.testing.assert_allclose(out, base[perm], rtol=RTOL, atol=ATOL)
+    assert np.array_equal(out, base[perm])
 
 
 @pytest.mark.parametrize("D", [32, 64])

@@ -33,7 +33,7 @@ def config_guard():
     _lib.config_set("sddmm.block_cols", 0)
     _lib.config_set("sddmm.rows_blocks", 0)
     _lib.config_set("sddmm.rows_wide", 0)
-    for key in ("sddmm.blocked", "sddmm.fast", "sddmm.buffer_loads", "sddmm.rows"):
+    for key in ("sddmm.blocked", "sddmm.fast", "sddmm.buffer_loads", "sddmm.rows", "sddmm.sorted_copy"):
         _lib.config_set(key, -1)
 
 
@@ -156,9 +156,11 @@ def test_column_blocked_edge_list(config_guard, F):
         assert np.array_equal(outs[0], plain)                        # one tile: same summation tree as the plain kernel
 
 
-def test_column_blocked_edge_list_keeps_the_callers_edge_order(config_guard):
+@pytest.mark.parametrize("sorted_copy", [0, 1])
+def test_column_blocked_edge_list_keeps_the_callers_edge_order(config_guard, sorted_copy):
     _lib.config_set("sddmm.blocked", 1)
     _lib.config_set("sddmm.block_cols", 500)
+    _lib.config_set("sddmm.sorted_copy", sorted_copy)              # 0: the edge-list kernel scatters its results
     coo = datasets.config_graph("c2-mini").tocoo()
     rng = np.random.default_rng(8)
     src = rng.integers(-8, 9, (coo.shape[1], 128)).astype(np.float32)
@@ -277,7 +279,7 @@ def test_default_plan_of_a_matrix_wider_than_one_column_block(config_guard, F):
     np.testing.assert_allclose(out, ref.sddmm_f64(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
 
 
-def test_row_runs_only_for_row_sorted_lists(config_guard):
+def test_which_lists_take_the_row_run_kernel(config_guard):
     _lib.config_set("sddmm.blocked", 1)
     _lib.config_set("sddmm.block_cols", 500)
     coo = datasets.config_graph("c2-mini").tocoo()
@@ -286,7 +288,12 @@ def test_row_runs_only_for_row_sorted_lists(config_guard):
     rng = np.random.default_rng(9)
     perm = rng.permutation(coo.nnz)
     shuffled = scipy.sparse.coo_matrix((coo.data[perm], (coo.row[perm], coo.col[perm])), shape=coo.shape)
+    # a list in any other order runs the same kernel over a sorted copy ...
+    text = _describe(VanillaSDDMMhip(shuffled), src, dst)
+    assert "row runs" in text and "sorted by row and column" in text
+    _lib.config_set("sddmm.sorted_copy", 0)                          # ... or, without one, the re-ordered edge list
     assert "column-blocked edge list" in _describe(VanillaSDDMMhip(shuffled), src, dst)
+    _lib.config_set("sddmm.sorted_copy", -1)
     # rows ascend but the columns inside a row do not: runs of one column block are no longer contiguous
     order = np.lexsort((rng.random(coo.nnz), coo.row))
     ragged = scipy.sparse.coo_matrix((coo.data[order], (coo.row[order], coo.col[order])), shape=coo.shape)
@@ -299,6 +306,36 @@ def test_row_runs_only_for_row_sorted_lists(config_guard):
     # 30 floats or several heads: neither blocked kernel applies
     src30, dst30 = datasets.sddmm_operands(coo, 30)
     assert "row runs" not in _describe(VanillaSDDMMhip(coo), src30, dst30)
+
+
+@pytest.mark.parametrize("F", [16, 32, 64, 128, 260, 512])
+def test_sorted_copy_of_a_list_in_any_order(config_guard, F):
+    """A shuffled list with edges listed twice and rows without edges: the plan sorts a copy by (row, column), the
+    row-run kernel works on the copy and a gather returns the results to the caller's positions.  Same kernel,
+    same tiles, same runs as for the sorted list, so the results are the sorted list's bit for bit."""
+    _lib.config_set("sddmm.block_cols", 700)
+    csr = datasets.config_graph("c2-mini").tocsr()
+    csr = scipy.sparse.vstack([csr[:100], scipy.sparse.csr_matrix((3, csr.shape[1]), dtype=csr.dtype), csr[100:]]).tocsr()
+    coo = csr.tocoo()
+    rng = np.random.default_rng(F)
+    twice = rng.integers(0, coo.nnz, 5000)
+    order = np.lexsort((np.concatenate([coo.col, coo.col[twice]]), np.concatenate([coo.row, coo.row[twice]])))
+    row = np.concatenate([coo.row, coo.row[twice]])[order]
+    col = np.concatenate([coo.col, coo.col[twice]])[order]
+    base = scipy.sparse.coo_matrix((np.ones(len(row), np.float32), (row, col)), shape=coo.shape)
+    perm = rng.permutation(len(row))
+    shuffled = scipy.sparse.coo_matrix((base.data[perm], (row[perm], col[perm])), shape=coo.shape)
+    src, dst = datasets.sddmm_operands(base, F)
+    text = _describe(VanillaSDDMMhip(shuffled), src, dst)
+    assert "sorted by row and column" in text
+    module = VanillaSDDMMhip(shuffled)
+    module.build([placeholder(src.shape), placeholder(dst.shape)], {}, {})
+    module.out_tvm.tensor.fill_(7.0)
+    ins = [nd.array(src, module.ctx), nd.array(dst, module.ctx)]
+    out = module.run(ins).asnumpy()
+    assert np.array_equal(out, _run_sddmm(base, src, dst)[perm])
+    np.testing.assert_allclose(out, ref.sddmm_f64(shuffled.row, shuffled.col, src, dst), rtol=RTOL, atol=ATOL)
+    assert np.array_equal(module.run(ins).asnumpy(), out)           # the plan's scratch carries nothing between calls
 
 
 def test_row_runs_on_awkward_structures(config_guard):
