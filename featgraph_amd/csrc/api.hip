@@ -435,6 +435,7 @@ int *config_slot(const char *key) {
   if (!strcmp(key, "sddmm.rows_blocks")) return &c.sddmm_rows_blocks;
   if (!strcmp(key, "sddmm.rows_wide")) return &c.sddmm_rows_wide;
   if (!strcmp(key, "sddmm.sorted_copy")) return &c.sddmm_sorted_copy;
+  if (!strcmp(key, "sddmm.regroup")) return &c.sddmm_regroup;
   if (!strcmp(key, "attention.blocks")) return &c.attention_blocks;
   return nullptr;
 }
@@ -935,7 +936,8 @@ int fg_config_set(const char *key, int32_t value) {
                     slot == &fg::config().sddmm_blocked ||
                     slot == &fg::config().spmm_buffer_loads || slot == &fg::config().sddmm_fast ||
                     slot == &fg::config().sddmm_buffer_loads || slot == &fg::config().sddmm_rows ||
-                    slot == &fg::config().spmm_multi || slot == &fg::config().sddmm_sorted_copy;
+                    slot == &fg::config().spmm_multi || slot == &fg::config().sddmm_sorted_copy ||
+                    slot == &fg::config().sddmm_regroup;
   // flags: 0 / 1 are explicit, anything negative restores the default;
   // sizes: 0 restores the default
   *slot = flag ? (value < 0 ? -1 : (value != 0)) : std::max(value, 0);

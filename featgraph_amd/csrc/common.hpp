@@ -28,7 +28,7 @@ struct Config {
   int spmm_multi = -1, spmm_multi_blocks = 0, spmm_multi_long = 0, spmm_tile_interleave = 0;
   int sddmm_group = 0, sddmm_batches = 0, sddmm_blocked = -1, sddmm_block_cols = 0;
   int sddmm_fast = -1, sddmm_buffer_loads = -1, sddmm_rows = -1, sddmm_rows_blocks = 0;
-  int attention_blocks = 0, sddmm_rows_wide = 0, sddmm_sorted_copy = -1;
+  int attention_blocks = 0, sddmm_rows_wide = 0, sddmm_sorted_copy = -1, sddmm_regroup = -1;
 };
 Config &config();
 
@@ -131,14 +131,18 @@ struct SddmmBlocks {
 struct SddmmSorted {
   int32_t *row_s = nullptr;    // [nnz] row ids in sorted order; freed once the row pointer is built
   int32_t *col_s = nullptr;    // [nnz] column ids in sorted order
-  int32_t *where = nullptr;    // [nnz] place of the caller's edge e in the sorted list
+  int32_t *where = nullptr;    // [nnz] place of the caller's edge e in the sorted list (null when `from` exists)
   float *results = nullptr;    // [nnz] the dot products in sorted order, between the kernel and the gather back
+  // The gather back as two block-local permutations (null: one gather through `where`)
+  uint16_t *a_local = nullptr;  // [nnz] place of sorted element i inside its block after step A
+  int32_t *from = nullptr;      // [nnz] place after step A of the j-th element of the caller's blocks
+  uint16_t *b_local = nullptr;  // [nnz] place of that element inside its block of the output
 };
 // Leaves *out empty (and returns FG_OK) for ids outside the matrix, sizes beyond int32 or when memory runs out.
 int sddmm_sorted_build(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_t *row, const int32_t *col,
                        SddmmSorted *out);
 void sddmm_sorted_free(SddmmSorted *s);
-// out[e] = s.results[s.where[e]]
+// out[e] = the result of the caller's edge e; s.results is left in another order
 int sddmm_unsort_launch(const SddmmSorted &s, int64_t nnz, float *out, hipStream_t stream);
 
 // num_col_partitions: 0 lets the library decide, 1 builds nothing, P > 1 builds P column blocks.

@@ -94,9 +94,157 @@ __global__ __launch_bounds__(256) void unsort_kernel(const float *sorted, const 
   }
 }
 
+// ---- the gather back in two local steps -------------------------------------------------------------------
+// out[e] = sorted[where[e]] reads 4 bytes from a random 128-byte line per edge.  The same permutation as two
+// steps that each permute only inside a block of kRegroup elements, through LDS, with coalesced stores:
+//   step A  block c of the sorted results is re-ordered, in place, by destination block:
+//           staged[c*K + a_local[i]] = sorted[i]
+//   step B  destination block b collects its elements, which lie in one short contiguous piece per source block
+//           (from[j] walks them), and puts each at its place: out[b*K + b_local[j]] = staged[from[j]]
+// so the only scattered accesses are step B's reads of pieces of K*K/nnz consecutive elements (9 on a list of
+// 115M edges: 16M pieces instead of 115M single reads).
+constexpr int kRegroup = 32768;        // elements per block: 128 KB of LDS
+constexpr int kRegroupThreads = 1024;
+
+__global__ void regroup_keys_kernel(const int32_t *pos, int64_t nnz, int block_bits, uint32_t *keys, int32_t *ids) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
+    keys[i] = (static_cast<uint32_t>(i / kRegroup) << block_bits) | static_cast<uint32_t>(pos[i] / kRegroup);
+    ids[i] = static_cast<int32_t>(i);
+  }
+}
+
+// order_a[p]: which sorted element lands at place p of the staged array
+__global__ void regroup_a_kernel(const int32_t *order_a, const int32_t *pos, int64_t nnz, uint16_t *a_local,
+                                 uint32_t *keys_b, int32_t *ids_b, uint16_t *b_local_of_place) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t p = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; p < nnz; p += stride) {
+    const int32_t i = order_a[p];
+    const int32_t e = pos[i];
+    a_local[i] = static_cast<uint16_t>(p % kRegroup);
+    keys_b[p] = static_cast<uint32_t>(e / kRegroup);
+    ids_b[p] = static_cast<int32_t>(p);
+    b_local_of_place[p] = static_cast<uint16_t>(e % kRegroup);
+  }
+}
+
+__global__ void regroup_b_kernel(const int32_t *from, const uint16_t *b_local_of_place, int64_t nnz, uint16_t *b_local) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t j = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; j < nnz; j += stride)
+    b_local[j] = b_local_of_place[from[j]];
+}
+
+// One workgroup per block of kRegroup elements: lds[local[j]] = in[from ? from[j] : j], then the block is stored
+// in order.  `local` is a permutation of the block's own places, so every LDS word is written once.
+template <bool GATHER>
+__global__ __launch_bounds__(kRegroupThreads) void regroup_kernel(const float *in, const int32_t *from,
+                                                                  const uint16_t *local, float *out, int64_t nnz) {
+  extern __shared__ float staged_block[];
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * kRegroup;
+  const int count = static_cast<int>(min(static_cast<int64_t>(kRegroup), nnz - base));
+  const int full = count & ~3;
+  for (int t = threadIdx.x * 4; t < full; t += kRegroupThreads * 4) {  // base is a multiple of 4 elements
+    const ushort4 l = *reinterpret_cast<const ushort4 *>(local + base + t);
+    float4 v;
+    if constexpr (GATHER) {
+      const int4 f = *reinterpret_cast<const int4 *>(from + base + t);
+      v = make_float4(in[f.x], in[f.y], in[f.z], in[f.w]);
+    } else {
+      v = *reinterpret_cast<const float4 *>(in + base + t);
+    }
+    staged_block[l.x] = v.x;
+    staged_block[l.y] = v.y;
+    staged_block[l.z] = v.z;
+    staged_block[l.w] = v.w;
+  }
+  for (int t = full + threadIdx.x; t < count; t += kRegroupThreads)
+    staged_block[local[base + t]] = in[GATHER ? static_cast<int64_t>(from[base + t]) : base + t];
+  __syncthreads();
+  if ((reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+    for (int t = threadIdx.x * 4; t < full; t += kRegroupThreads * 4)
+      *reinterpret_cast<float4 *>(out + base + t) = *reinterpret_cast<const float4 *>(staged_block + t);
+    for (int t = full + threadIdx.x; t < count; t += kRegroupThreads) out[base + t] = staged_block[t];
+  } else {
+    for (int t = threadIdx.x; t < count; t += kRegroupThreads) out[base + t] = staged_block[t];
+  }
+}
+
+// Builds a_local / from / b_local from pos[i], the caller's place of sorted element i.
+hipError_t regroup_build(const int32_t *pos, int64_t nnz, SddmmSorted *out) {
+  const size_t n = static_cast<size_t>(nnz);
+  const int64_t n_blocks = (nnz + kRegroup - 1) / kRegroup;
+  int block_bits = 1;
+  while ((int64_t{1} << block_bits) < n_blocks) ++block_bits;
+  if (2 * block_bits > 32) return hipSuccess;  // beyond 2^31 edges anyway
+  const int grid = static_cast<int>(std::min<int64_t>((nnz + 255) / 256, 65536));
+  uint32_t *keys = nullptr, *keys_sorted = nullptr;
+  int32_t *ids = nullptr, *order_a = nullptr;
+  uint16_t *b_local_of_place = nullptr;
+  void *tmp = nullptr;
+  size_t tmp_a = 0, tmp_b = 0;
+  hipError_t err = hipMalloc(&keys, n * sizeof(uint32_t));
+  if (err == hipSuccess) err = hipMalloc(&keys_sorted, n * sizeof(uint32_t));
+  if (err == hipSuccess) err = hipMalloc(&ids, n * sizeof(int32_t));
+  if (err == hipSuccess) err = hipMalloc(&order_a, n * sizeof(int32_t));
+  if (err == hipSuccess) err = hipMalloc(&b_local_of_place, n * sizeof(uint16_t));
+  if (err == hipSuccess) err = hipMalloc(&out->a_local, n * sizeof(uint16_t));
+  if (err == hipSuccess) err = hipMalloc(&out->b_local, n * sizeof(uint16_t));
+  if (err == hipSuccess) err = hipMalloc(&out->from, n * sizeof(int32_t));
+  if (err == hipSuccess)
+    err = hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_a, keys, keys_sorted, ids, order_a, static_cast<int>(nnz), 0,
+                                             2 * block_bits, nullptr);
+  if (err == hipSuccess)
+    err = hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_b, keys, keys_sorted, ids, out->from, static_cast<int>(nnz), 0,
+                                             block_bits, nullptr);
+  if (err == hipSuccess) err = hipMalloc(&tmp, std::max<size_t>(std::max(tmp_a, tmp_b), 1));
+  if (err == hipSuccess) {
+    regroup_keys_kernel<<<dim3(grid), dim3(256)>>>(pos, nnz, block_bits, keys, ids);
+    err = hipGetLastError();
+  }
+  if (err == hipSuccess)  // source block above destination block; stable, so a piece keeps the sorted order
+    err = hipcub::DeviceRadixSort::SortPairs(tmp, tmp_a, keys, keys_sorted, ids, order_a, static_cast<int>(nnz), 0,
+                                             2 * block_bits, nullptr);
+  if (err == hipSuccess) {
+    regroup_a_kernel<<<dim3(grid), dim3(256)>>>(order_a, pos, nnz, out->a_local, keys, ids, b_local_of_place);
+    err = hipGetLastError();
+  }
+  if (err == hipSuccess)  // by destination block; stable, so a block's pieces come by ascending place
+    err = hipcub::DeviceRadixSort::SortPairs(tmp, tmp_b, keys, keys_sorted, ids, out->from, static_cast<int>(nnz), 0,
+                                             block_bits, nullptr);
+  if (err == hipSuccess) {
+    regroup_b_kernel<<<dim3(grid), dim3(256)>>>(out->from, b_local_of_place, nnz, out->b_local);
+    err = hipGetLastError();
+  }
+  if (err == hipSuccess) err = hipDeviceSynchronize();
+  if (err == hipSuccess) {
+    err = hipFuncSetAttribute(reinterpret_cast<const void *>(&regroup_kernel<false>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kRegroup * sizeof(float));
+    if (err == hipSuccess)
+      err = hipFuncSetAttribute(reinterpret_cast<const void *>(&regroup_kernel<true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kRegroup * sizeof(float));
+  }
+  if (keys) (void)hipFree(keys);
+  if (keys_sorted) (void)hipFree(keys_sorted);
+  if (ids) (void)hipFree(ids);
+  if (order_a) (void)hipFree(order_a);
+  if (b_local_of_place) (void)hipFree(b_local_of_place);
+  if (tmp) (void)hipFree(tmp);
+  if (err != hipSuccess) {  // the one-step gather still works
+    if (out->a_local) (void)hipFree(out->a_local);
+    if (out->b_local) (void)hipFree(out->b_local);
+    if (out->from) (void)hipFree(out->from);
+    out->a_local = out->b_local = nullptr;
+    out->from = nullptr;
+  }
+  return err;
+}
+
 }  // namespace
 
 void sddmm_sorted_free(SddmmSorted *s) {
+  if (s->a_local) (void)hipFree(s->a_local);
+  if (s->b_local) (void)hipFree(s->b_local);
+  if (s->from) (void)hipFree(s->from);
   if (s->row_s) (void)hipFree(s->row_s);
   if (s->col_s) (void)hipFree(s->col_s);
   if (s->where) (void)hipFree(s->where);
@@ -152,9 +300,20 @@ int sddmm_sorted_build(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_
   if (keys) (void)hipFree(keys);
   if (keys_sorted) (void)hipFree(keys_sorted);
   if (ids) (void)hipFree(ids);
+  if (tmp) (void)hipFree(tmp);
+  if (err == hipSuccess && !bad && config().sddmm_regroup != 0) {
+    const hipError_t e2 = regroup_build(pos, nnz, out);
+    if (e2 == hipErrorOutOfMemory)
+      (void)hipGetLastError();
+    else
+      err = e2;
+    if (out->from) {  // the one-step gather's index is not needed then
+      (void)hipFree(out->where);
+      out->where = nullptr;
+    }
+  }
   if (pos) (void)hipFree(pos);
   if (flag) (void)hipFree(flag);
-  if (tmp) (void)hipFree(tmp);
   if (err != hipSuccess || bad) {
     sddmm_sorted_free(out);
     if (err == hipSuccess) return FG_OK;
@@ -169,6 +328,16 @@ int sddmm_sorted_build(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_
 
 int sddmm_unsort_launch(const SddmmSorted &s, int64_t nnz, float *out, hipStream_t stream) {
   if (nnz == 0) return FG_OK;
+  if (s.from) {
+    const unsigned blocks = static_cast<unsigned>((nnz + kRegroup - 1) / kRegroup);
+    const size_t lds = kRegroup * sizeof(float);
+    // step A works in place: a workgroup has read its whole block before it stores the first element
+    regroup_kernel<false><<<dim3(blocks), dim3(kRegroupThreads), lds, stream>>>(s.results, nullptr, s.a_local, s.results, nnz);
+    FG_HIP_TRY(hipGetLastError());
+    regroup_kernel<true><<<dim3(blocks), dim3(kRegroupThreads), lds, stream>>>(s.results, s.from, s.b_local, out, nnz);
+    FG_HIP_TRY(hipGetLastError());
+    return FG_OK;
+  }
   const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((nnz + 1023) / 1024, 1 << 20));
   unsort_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(s.results, s.where, out, nnz);
   FG_HIP_TRY(hipGetLastError());

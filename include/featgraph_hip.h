@@ -190,11 +190,12 @@ FG_API int fg_sddmm_coo_general_f32(int64_t nnz, const int32_t *row, const int32
  * inside every row ((2 * n_cols/16384 + 3) * n_rows int32).  For a list in any
  * other order it sorts a copy of the list by (row, column) (one device radix
  * sort, stable), builds the same tables over the copy, and keeps the copy's
- * column ids, every edge's place in the copy and room for the results in that
- * order: 12 bytes per edge.  A call then runs the same kernel as for a sorted
- * list and gathers the results back, so they are always written in the
- * caller's edge order (there is no edge_mapping to apply) and equal the sorted
- * list's bit for bit.  Because the results pass through memory that the plan
+ * column ids, room for the results in that order and the routing that brings
+ * them back to the caller's order in two steps that each permute inside blocks
+ * of 32768 results ("sddmm.regroup" = 0: one gather instead): 16 bytes per
+ * edge.  A call then runs the same kernel as for a sorted list and returns the
+ * results, so they are always written in the caller's edge order (there is no
+ * edge_mapping to apply) and equal the sorted list's bit for bit.  Because the results pass through memory that the plan
  * owns, two calls on ONE plan of an unsorted list must not overlap in time.
  * Rows that ascend while their columns do not, lists with ids outside the
  * matrix and "sddmm.sorted_copy" = 0 fall back to a copy re-ordered by column
@@ -371,7 +372,9 @@ FG_API int64_t fg_probe_store_rows_f32(float *out, int64_t n_out_rows, int32_t r
  * half the width for feature rows of 128 floats and more; by default 2 when a
  * (row, pass) run then still holds 8 edges on average),
  * "sddmm.sorted_copy" (0/1: whether a plan over a list that is not row-sorted
- * works on a sorted copy, read at plan creation; default 1),
+ * works on a sorted copy, read at plan creation; default 1), "sddmm.regroup"
+ * (0/1: whether such a plan returns the results through two block-local
+ * permutations or one gather, read at plan creation; default 1),
  * "attention.blocks" (grid size of the fused attention kernel; by default one
  * vertex row per wave when a row is 1 KB or more, else 65536 workgroups that
  * walk the rows).  Value 0 restores the default of a size; for the 0/1 flags a

@@ -33,7 +33,7 @@ def config_guard():
     _lib.config_set("sddmm.block_cols", 0)
     _lib.config_set("sddmm.rows_blocks", 0)
     _lib.config_set("sddmm.rows_wide", 0)
-    for key in ("sddmm.blocked", "sddmm.fast", "sddmm.buffer_loads", "sddmm.rows", "sddmm.sorted_copy"):
+    for key in ("sddmm.blocked", "sddmm.fast", "sddmm.buffer_loads", "sddmm.rows", "sddmm.sorted_copy", "sddmm.regroup"):
         _lib.config_set(key, -1)
 
 
@@ -308,12 +308,15 @@ def test_which_lists_take_the_row_run_kernel(config_guard):
     assert "row runs" not in _describe(VanillaSDDMMhip(coo), src30, dst30)
 
 
+@pytest.mark.parametrize("regroup", [1, 0])
 @pytest.mark.parametrize("F", [16, 32, 64, 128, 260, 512])
-def test_sorted_copy_of_a_list_in_any_order(config_guard, F):
+def test_sorted_copy_of_a_list_in_any_order(config_guard, F, regroup):
     """A shuffled list with edges listed twice and rows without edges: the plan sorts a copy by (row, column), the
-    row-run kernel works on the copy and a gather returns the results to the caller's positions.  Same kernel,
-    same tiles, same runs as for the sorted list, so the results are the sorted list's bit for bit."""
+    row-run kernel works on the copy and the results return to the caller's positions, through two block-local
+    permutations or (regroup = 0) one gather.  Same kernel, same tiles, same runs as for the sorted list, so the
+    results are the sorted list's bit for bit."""
     _lib.config_set("sddmm.block_cols", 700)
+    _lib.config_set("sddmm.regroup", regroup)
     csr = datasets.config_graph("c2-mini").tocsr()
     csr = scipy.sparse.vstack([csr[:100], scipy.sparse.csr_matrix((3, csr.shape[1]), dtype=csr.dtype), csr[100:]]).tocsr()
     coo = csr.tocoo()
@@ -336,6 +339,33 @@ def test_sorted_copy_of_a_list_in_any_order(config_guard, F):
     assert np.array_equal(out, _run_sddmm(base, src, dst)[perm])
     np.testing.assert_allclose(out, ref.sddmm_f64(shuffled.row, shuffled.col, src, dst), rtol=RTOL, atol=ATOL)
     assert np.array_equal(module.run(ins).asnumpy(), out)           # the plan's scratch carries nothing between calls
+    # through the C ABI into an output that is 4-byte but not 16-byte aligned
+    import torch
+    room = torch.full((len(row) + 1,), 7.0, dtype=torch.float32, device=module.ctx)
+    stream = torch.cuda.current_stream(module.ctx).cuda_stream
+    _lib.check(_lib.lib().fg_sddmm_coo_plan_f32(module._plan, ins[0].tensor.data_ptr(), ins[1].tensor.data_ptr(),
+                                                room.data_ptr() + 4, 1, F, stream))
+    assert np.array_equal(room[1:].cpu().numpy(), out) and float(room[0]) == 7.0
+
+
+@pytest.mark.parametrize("nnz", [1, 3, 5, 32767, 32768, 32769, 65539])
+def test_sorted_copy_sizes_around_the_regrouping_block(config_guard, nnz):
+    """Lists of one edge, fewer than four, and one off either side of the 32768-element blocks that the results
+    are regrouped in; exact on integer operands."""
+    _lib.config_set("sddmm.blocked", 1)
+    _lib.config_set("sddmm.block_cols", 40)
+    rng = np.random.default_rng(nnz)
+    n_rows, n_cols, F = 300, 257, 64
+    row = rng.integers(0, n_rows, nnz).astype(np.int32)
+    col = rng.integers(0, n_cols, nnz).astype(np.int32)
+    row[0], row[-1] = n_rows - 1, 0                                   # never row-sorted, except the list of one edge
+    coo = scipy.sparse.coo_matrix((np.ones(nnz, np.float32), (row, col)), shape=(n_rows, n_cols))
+    src = rng.integers(-8, 9, (n_cols, F)).astype(np.float32)
+    dst = rng.integers(-8, 9, (n_rows, F)).astype(np.float32)
+    if nnz > 1:
+        assert "sorted by row and column" in _describe(VanillaSDDMMhip(coo), src, dst)
+    want = (src[col].astype(np.int64) * dst[row].astype(np.int64)).sum(-1).astype(np.float32)
+    assert np.array_equal(_run_sddmm(coo, src, dst), want)
 
 
 def test_row_runs_on_awkward_structures(config_guard):
