@@ -223,7 +223,8 @@ int multi_merge(const fg_spmm_plan *plan, int tile) {
 int multi_build(fg_spmm_plan *p) {
   if (fg::config().spmm_multi == 0 || !p->seg || !p->row_order || p->n_rows == 0) return FG_OK;
   const int32_t n = static_cast<int32_t>(p->n_rows);
-  if (int rc = fg::multi_runs_build(p->seg, p->row_order, n, p->n_blocks, p->n_blocks, &p->multi_whole)) return rc;
+  if (int rc = fg::multi_runs_build(p->seg, p->row_order, p->indices, p->nnz, n, p->n_blocks, p->n_blocks, &p->multi_whole))
+    return rc;
   if (p->n_blocks < 2) return FG_OK;
   const int tiles[3] = {16, 32, 64};
   for (int t = 0; t < 3; ++t) {
@@ -240,7 +241,8 @@ int multi_build(fg_spmm_plan *p) {
         shared = true;
       }
     if (!shared)
-      if (int rc = fg::multi_runs_build(p->seg, p->row_order, n, p->n_blocks, merge, &p->multi_tile[t])) return rc;
+      if (int rc = fg::multi_runs_build(p->seg, p->row_order, p->indices, p->nnz, n, p->n_blocks, merge, &p->multi_tile[t]))
+        return rc;
   }
   return FG_OK;
 }
@@ -286,6 +288,10 @@ int multi_interleave(int n_tiles) {
 }
 
 int multi_run(const fg_spmm_plan *plan, const fg::MultiRuns *runs, fg::SpmmArgs a, hipStream_t st) {
+  if (runs->ids_p) {  // the records index the re-laid ids and say where each run's values start in the CSR array
+    a.indices = runs->ids_p;
+    a.vals_by_csr = 1;
+  }
   const int tile = fg::spmm_multi_tile(a.F);
   const int n_tiles = (a.F + tile - 1) / tile;
   const int64_t n = plan->n_rows;
@@ -425,6 +431,7 @@ int *config_slot(const char *key) {
   if (!strcmp(key, "spmm.multi_blocks")) return &c.spmm_multi_blocks;
   if (!strcmp(key, "spmm.multi_long")) return &c.spmm_multi_long;
   if (!strcmp(key, "spmm.tile_interleave")) return &c.spmm_tile_interleave;
+  if (!strcmp(key, "spmm.relay")) return &c.spmm_relay;
   if (!strcmp(key, "sddmm.group")) return &c.sddmm_group;
   if (!strcmp(key, "sddmm.batches")) return &c.sddmm_batches;
   if (!strcmp(key, "sddmm.blocked")) return &c.sddmm_blocked;
@@ -937,7 +944,7 @@ int fg_config_set(const char *key, int32_t value) {
                     slot == &fg::config().spmm_buffer_loads || slot == &fg::config().sddmm_fast ||
                     slot == &fg::config().sddmm_buffer_loads || slot == &fg::config().sddmm_rows ||
                     slot == &fg::config().spmm_multi || slot == &fg::config().sddmm_sorted_copy ||
-                    slot == &fg::config().sddmm_regroup;
+                    slot == &fg::config().sddmm_regroup || slot == &fg::config().spmm_relay;
   // flags: 0 / 1 are explicit, anything negative restores the default;
   // sizes: 0 restores the default
   *slot = flag ? (value < 0 ? -1 : (value != 0)) : std::max(value, 0);

@@ -28,7 +28,7 @@ struct Config {
   int spmm_multi = -1, spmm_multi_blocks = 0, spmm_multi_long = 0, spmm_tile_interleave = 0;
   int sddmm_group = 0, sddmm_batches = 0, sddmm_blocked = -1, sddmm_block_cols = 0;
   int sddmm_fast = -1, sddmm_buffer_loads = -1, sddmm_rows = -1, sddmm_rows_blocks = 0;
-  int attention_blocks = 0, sddmm_rows_wide = 0, sddmm_sorted_copy = -1, sddmm_regroup = -1;
+  int attention_blocks = 0, sddmm_rows_wide = 0, sddmm_sorted_copy = -1, sddmm_regroup = -1, spmm_relay = -1;
 };
 Config &config();
 
@@ -65,6 +65,9 @@ struct SpmmArgs {
   int32_t long_runs = 0;    // the first long_runs records are long runs: one wave each, in the first
   int32_t long_blocks = 0;  // long_blocks workgroups of the grid
   int32_t interleave_tiles = 1;  // this many tiles alternate workgroup by workgroup along grid.x; the rest along grid.y
+  // records over a re-laid copy of the ids (MultiRuns::ids_p): `indices` is that copy, and a run's values start
+  // at the CSR position in the record's fourth entry
+  int32_t vals_by_csr = 0;
 };
 
 struct SpmmShape {
@@ -85,9 +88,16 @@ struct MultiRuns {
   int32_t merge = 0;    // column blocks of the bounds table per pass
   int32_t passes = 0;
   int32_t *long_runs = nullptr;  // [passes], host, owned: how many of a pass's records are long runs
+  // With several passes: the column ids laid out in the order the records are visited (pass after pass, inside a
+  // pass by descending run length), every run starting on a multiple of four entries, so that a pass reads its
+  // ids front to back instead of one short piece of the CSR array per run.  The records then hold
+  // {first, last + 1 in this layout, row, first in the CSR arrays}.  Null: the records index the CSR arrays.
+  int32_t *ids_p = nullptr;   // [relaid_n], device, owned
+  int64_t relaid_n = 0;
 };
-int multi_runs_build(const int32_t *seg, const int32_t *row_order, int32_t n_rows, int32_t n_blocks, int32_t merge,
-                     MultiRuns *out);
+// indices: the CSR column ids (for the re-laid copy; null builds none)
+int multi_runs_build(const int32_t *seg, const int32_t *row_order, const int32_t *indices, int64_t nnz, int32_t n_rows,
+                     int32_t n_blocks, int32_t merge, MultiRuns *out);
 void multi_runs_free(MultiRuns *r);
 int spmm_multi_tile(int32_t F);
 bool spmm_multi_applies(const SpmmArgs &a);

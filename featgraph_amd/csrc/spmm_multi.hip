@@ -128,6 +128,7 @@ __device__ __forceinline__ void spmm_long_runs(const SpmmArgs &a, const FeatRows
   const int f1 = (a.tile_base + tile) * TW + lane;  // the float this lane sums
   const bool owner = lane < TW && f1 < a.F;
 
+  int vo = 0;  // from a nonzero's place in the id array to its place in the value array
   auto load_ids = [&](int e, int rem, Ids &d) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
@@ -135,7 +136,7 @@ __device__ __forceinline__ void spmm_long_runs(const SpmmArgs &a, const FeatRows
       d.v[q] = 0.0f;
       if (64 * q + lane < rem) {
         d.c[q] = a.indices[e + 64 * q + lane];
-        d.v[q] = a.w[e + 64 * q + lane];
+        d.v[q] = a.w[e + vo + 64 * q + lane];
       }
     }
   };
@@ -182,6 +183,7 @@ __device__ __forceinline__ void spmm_long_runs(const SpmmArgs &a, const FeatRows
     const int4 rec = a.runs[it];
     const int lo = rec.x, hi = rec.y, row = rec.z;
     if (hi <= lo) continue;
+    vo = a.vals_by_csr ? rec.w - rec.x : 0;
     float acc = 0.0f;
     float4 xa[R], xb[R];
     Ids ids_a;
@@ -245,8 +247,10 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_multi_kernel(const SpmmArg
   int item = __builtin_amdgcn_readfirstlane(
       static_cast<int>((bx - a.long_blocks) * kWavesPerBlock + (threadIdx.x >> 6)));
 
-  auto bounds = [&](int it, int &lo, int &hi, int &row) {
-    lo = hi = 0;
+  const bool by_csr = a.vals_by_csr != 0;
+  // vo: from a nonzero's place in the id array to its place in the value array
+  auto bounds = [&](int it, int &lo, int &hi, int &row, int &vo) {
+    lo = hi = vo = 0;
     row = -1;
     const int pos = a.long_runs + it * NG + g;
     if (it < n_items && pos < n) {
@@ -254,11 +258,12 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_multi_kernel(const SpmmArg
       lo = r.x;
       hi = r.y;
       row = r.z;
+      if (by_csr) vo = r.w - r.x;
     }
   };
   // this lane's four ids / values of the batch that starts at nonzero e, of which the group has `rem` left;
   // slots past the end hold column id 0 (a valid row to gather from, never added)
-  auto load_ids = [&](int e, int rem, Ids &d) {
+  auto load_ids = [&](int e, int rem, int vo, Ids &d) {
     const int k0 = 4 * gl;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
@@ -267,7 +272,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_multi_kernel(const SpmmArg
     }
     if (k0 + 3 < rem) {
       const Int4U ci = *reinterpret_cast<const Int4U *>(a.indices + e + k0);
-      const Float4U vi = *reinterpret_cast<const Float4U *>(a.w + e + k0);
+      const Float4U vi = *reinterpret_cast<const Float4U *>(a.w + e + vo + k0);
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         d.c[k] = ci.v[k];
@@ -278,28 +283,28 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_multi_kernel(const SpmmArg
       for (int k = 0; k < 4; ++k)
         if (k0 + k < rem) {
           d.c[k] = a.indices[e + k0 + k];
-          d.v[k] = a.w[e + k0 + k];
+          d.v[k] = a.w[e + vo + k0 + k];
         }
     }
   };
-  auto first_ids = [&](int lo, int hi, int row, Ids &d, float4 &acc) {
-    load_ids(lo, hi - lo, d);
+  auto first_ids = [&](int lo, int hi, int row, int vo, Ids &d, float4 &acc) {
+    load_ids(lo, hi - lo, vo, d);
     acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     if (carry && hi > lo && fok) acc = *reinterpret_cast<const float4 *>(a.out + static_cast<int64_t>(row) * F + f0);
   };
 
-  int lo_a, hi_a, row_a, lo_b, hi_b, row_b;
+  int lo_a, hi_a, row_a, vo_a, lo_b, hi_b, row_b, vo_b;
   Ids ids_a;
   float4 acc_a;
-  bounds(item, lo_a, hi_a, row_a);
-  first_ids(lo_a, hi_a, row_a, ids_a, acc_a);
-  bounds(item + n_waves, lo_b, hi_b, row_b);
+  bounds(item, lo_a, hi_a, row_a, vo_a);
+  first_ids(lo_a, hi_a, row_a, vo_a, ids_a, acc_a);
+  bounds(item + n_waves, lo_b, hi_b, row_b, vo_b);
 
   while (item < n_items) {
-    int lo_c, hi_c, row_c, e = lo_a, rem = hi_a - lo_a;  // rem: nonzeros this group still has
+    int lo_c, hi_c, row_c, vo_c, e = lo_a, rem = hi_a - lo_a;  // rem: nonzeros this group still has
     Ids ids_b;
     float4 acc_b;
-    bounds(item + 2 * n_waves, lo_c, hi_c, row_c);
+    bounds(item + 2 * n_waves, lo_c, hi_c, row_c, vo_c);
     bool next_asked = false;
 
     while (__builtin_amdgcn_ballot_w64(rem > 0) != 0) {
@@ -317,9 +322,9 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_multi_kernel(const SpmmArg
             }
           });
           if (l0 == 0) {  // behind the batch's first gathers: the next item's first ids (once), this item's next batch
-            if (!next_asked) first_ids(lo_b, hi_b, row_b, ids_b, acc_b);
+            if (!next_asked) first_ids(lo_b, hi_b, row_b, vo_b, ids_b, acc_b);
             next_asked = true;
-            load_ids(e + B, rem - B, ids_n);
+            load_ids(e + B, rem - B, vo_a, ids_n);
           }
           static_for(std::make_integer_sequence<int, SC>{}, [&](auto u) {
             constexpr int l = l0 + decltype(u)::value;
@@ -342,18 +347,20 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_multi_kernel(const SpmmArg
       e += B;
       rem -= B;
     }
-    if (!next_asked) first_ids(lo_b, hi_b, row_b, ids_b, acc_b);  // no group had a nonzero here
+    if (!next_asked) first_ids(lo_b, hi_b, row_b, vo_b, ids_b, acc_b);  // no group had a nonzero here
     if (fok && row_a >= 0 && (hi_a > lo_a || !carry))
       *reinterpret_cast<float4 *>(a.out + static_cast<int64_t>(row_a) * F + f0) = acc_a;
 
     lo_a = lo_b;
     hi_a = hi_b;
     row_a = row_b;
+    vo_a = vo_b;
     ids_a = ids_b;
     acc_a = acc_b;
     lo_b = lo_c;
     hi_b = hi_c;
     row_b = row_c;
+    vo_b = vo_c;
     item += n_waves;
   }
 }
@@ -401,12 +408,75 @@ __global__ void run_records_kernel(const int32_t *seg_lo, const int32_t *seg_hi,
   }
 }
 
+// Entries that a record's run takes in the re-laid arrays: its length rounded up to a multiple of four.
+__global__ void padded_lengths_kernel(const int4 *rec, int64_t n, int32_t *len) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) len[i] = (max(rec[i].y - rec[i].x, 0) + 3) & ~3;
+}
+
+// One wave per record: copies the run's column ids to its new place and rewrites the record as
+// {first, last + 1 in the new layout, row, first in the CSR arrays}.
+__global__ void relay_ids_kernel(int4 *rec, const int32_t *first_p, int64_t n, const int32_t *indices, int32_t *ids_p) {
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int64_t waves = static_cast<int64_t>(gridDim.x) * (blockDim.x / kWaveSize);
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWaveSize) + threadIdx.x / kWaveSize; i < n; i += waves) {
+    const int4 r = rec[i];
+    const int len = max(r.y - r.x, 0), to = first_p[i];
+    for (int k = lane; k < len; k += kWaveSize) ids_p[to + k] = indices[r.x + k];
+    if (lane == 0) rec[i] = make_int4(to, to + len, r.z, r.x);
+  }
+}
+
+// The re-laid copy of the ids for a table of several passes.  Failure to allocate leaves the table as it is.
+hipError_t relay_build(const int32_t *indices, int64_t nnz, int64_t n_rec, MultiRuns *out) {
+  if (nnz + 3 * n_rec >= 0x7fffffffLL) return hipSuccess;
+  int32_t *len = nullptr, *first_p = nullptr;
+  void *tmp = nullptr;
+  size_t tmp_bytes = 0;
+  int32_t last[2] = {0, 0};
+  hipError_t err = hipMalloc(&len, n_rec * sizeof(int32_t));
+  if (err == hipSuccess) err = hipMalloc(&first_p, n_rec * sizeof(int32_t));
+  if (err == hipSuccess)
+    err = hipcub::DeviceScan::ExclusiveSum(nullptr, tmp_bytes, len, first_p, static_cast<int>(n_rec), nullptr);
+  if (err == hipSuccess) err = hipMalloc(&tmp, tmp_bytes ? tmp_bytes : 1);
+  const unsigned grid = static_cast<unsigned>((n_rec + 255) / 256);
+  if (err == hipSuccess) {
+    padded_lengths_kernel<<<dim3(grid), dim3(256)>>>(out->rec, n_rec, len);
+    err = hipGetLastError();
+  }
+  if (err == hipSuccess)
+    err = hipcub::DeviceScan::ExclusiveSum(tmp, tmp_bytes, len, first_p, static_cast<int>(n_rec), nullptr);
+  if (err == hipSuccess) err = hipMemcpy(&last[0], first_p + n_rec - 1, sizeof(int32_t), hipMemcpyDeviceToHost);
+  if (err == hipSuccess) err = hipMemcpy(&last[1], len + n_rec - 1, sizeof(int32_t), hipMemcpyDeviceToHost);
+  const int64_t total = static_cast<int64_t>(last[0]) + last[1];
+  int32_t *ids_p = nullptr;
+  if (err == hipSuccess) err = hipMalloc(&ids_p, std::max<int64_t>(total, 1) * sizeof(int32_t));
+  if (err == hipSuccess) err = hipMemset(ids_p, 0, std::max<int64_t>(total, 1) * sizeof(int32_t));  // padding: column 0
+  if (err == hipSuccess) {
+    const unsigned g2 = static_cast<unsigned>(std::min<int64_t>((n_rec + 3) / 4, 65536));
+    relay_ids_kernel<<<dim3(g2), dim3(256)>>>(out->rec, first_p, n_rec, indices, ids_p);
+    err = hipGetLastError();
+  }
+  if (err == hipSuccess) err = hipDeviceSynchronize();
+  if (len) (void)hipFree(len);
+  if (first_p) (void)hipFree(first_p);
+  if (tmp) (void)hipFree(tmp);
+  if (err != hipSuccess) {
+    if (ids_p) (void)hipFree(ids_p);
+    return err;  // the records are rewritten only by the last kernel: on failure before it they still index the CSR arrays
+  }
+  out->ids_p = ids_p;
+  out->relaid_n = total;
+  return hipSuccess;
+}
+
 }  // namespace
 
 int spmm_multi_tile(int32_t F) { return F <= 16 ? 16 : F <= 32 ? 32 : 64; }
 
 void multi_runs_free(MultiRuns *r) {
   if (r->rec) (void)hipFree(r->rec);
+  if (r->ids_p) (void)hipFree(r->ids_p);
   delete[] r->long_runs;
   *r = MultiRuns();
 }
@@ -414,8 +484,8 @@ void multi_runs_free(MultiRuns *r) {
 // One record {first nonzero, one past the last, row id} per (pass, row): pass p covers the column blocks
 // p * merge .. p * merge + merge - 1 of the bounds table, and inside a pass the rows come by descending run
 // length (ties in the table's order), so the rows that share a wave finish together.
-int multi_runs_build(const int32_t *seg, const int32_t *row_order, int32_t n_rows, int32_t n_blocks, int32_t merge,
-                     MultiRuns *out) {
+int multi_runs_build(const int32_t *seg, const int32_t *row_order, const int32_t *indices, int64_t nnz, int32_t n_rows,
+                     int32_t n_blocks, int32_t merge, MultiRuns *out) {
   *out = MultiRuns();
   if (n_rows == 0 || n_blocks < 1) return FG_OK;
   merge = std::max(1, std::min(merge, n_blocks));
@@ -472,6 +542,15 @@ int multi_runs_build(const int32_t *seg, const int32_t *row_order, int32_t n_row
   }
   out->merge = merge;
   out->passes = passes;
+  if (passes >= 2 && indices && config().spmm_relay != 0) {
+    const hipError_t e2 = relay_build(indices, nnz, static_cast<int64_t>(passes) * n_rows, out);
+    if (e2 == hipErrorOutOfMemory) {
+      (void)hipGetLastError();
+    } else if (e2 != hipSuccess) {
+      multi_runs_free(out);
+      return fail(FG_EHIP, "SpMM re-laid column ids: %s", hipGetErrorString(e2));
+    }
+  }
   return FG_OK;
 }
 

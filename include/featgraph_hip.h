@@ -361,6 +361,9 @@ FG_API int64_t fg_probe_store_rows_f32(float *out, int64_t n_out_rows, int32_t r
  * "spmm.multi_long" (run length from which a run gets a wave of its own,
  * default 512; read at plan creation), "spmm.tile_interleave" (feature tiles
  * whose workgroups alternate inside one launch of that kernel: 1 or 2, default 2),
+ * "spmm.relay" (0/1: whether the plan keeps, per pass layout of that kernel, a
+ * copy of the column ids in the order the passes visit them; read at plan
+ * creation; default 1),
  * "sddmm.blocked" (0/1: never / always build and use column blocks, read at
  * plan creation), "sddmm.block_cols" (columns per block, read at plan creation),
  * "sddmm.group" (lanes per dot product: 1..16),

@@ -39,7 +39,7 @@ def config_guard():
                 "spmm.multi_blocks", "spmm.multi_long", "spmm.tile_interleave"):
         _lib.config_set(key, 0)
     for key in ("spmm.sorted", "spmm.blocked", "spmm.pipeline",
-                "spmm.buffer_loads", "spmm.multi"):
+                "spmm.buffer_loads", "spmm.multi", "spmm.relay"):
         _lib.config_set(key, -1)
 
 
@@ -324,7 +324,10 @@ def test_rows_per_wave_kernel_on_degenerate_rows(config_guard, long_run):
     indices = np.concatenate([np.sort(rng.integers(0, 500, l)) for l in lens]).astype(np.int32)
     vals = rng.random(indptr[-1], dtype=np.float32)
     adj = scipy.sparse.csr_matrix((vals, indices, indptr), shape=(len(lens), 500))
-    for blocked, block_cols, grid, buf in ((0, 0, 0, -1), (1, 64, 0, -1), (1, 64, 1, 0), (0, 0, 1, 0)):
+    # relay 0: the records index the CSR arrays instead of a copy of the ids in visiting order
+    for blocked, block_cols, grid, buf, relay in ((0, 0, 0, -1, -1), (1, 64, 0, -1, -1), (1, 64, 0, -1, 0),
+                                                 (1, 64, 1, 0, -1), (1, 64, 1, 0, 0), (0, 0, 1, 0, -1)):
+        _lib.config_set("spmm.relay", relay)
         _lib.config_set("spmm.blocked", blocked)
         _lib.config_set("spmm.block_cols", block_cols)
         _lib.config_set("spmm.multi_blocks", grid)     # one workgroup: every wave walks several items
@@ -519,6 +522,7 @@ def test_random_structures_bit_exact_under_random_schedules(config_guard, seed):
     _lib.config_set("spmm.block_cols", int(rng.choice([1, 5, 64, 300, 1 << 20])))
     _lib.config_set("spmm.multi_long", int(rng.choice([0, 4, 64, 700])))
     _lib.config_set("spmm.multi_blocks", int(rng.choice([0, 1, 2])))
+    _lib.config_set("spmm.relay", int(seed % 3 != 0))
     module = VanillaSpMMhip(adj)
     for F in rng.choice([1, 3, 4, 8, 12, 16, 24, 32, 48, 64, 100, 128, 192, 260], 5, replace=False):
         feat = rng.standard_normal((n_cols, int(F))).astype(np.float32)
