@@ -122,7 +122,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--feat-len", type=int, default=64, help="feature length of the timed step")
     ap.add_argument("--graph", default="c2", help="named synthetic configuration (featgraph_amd.datasets.CONFIGS)")
-    ap.add_argument("--only", choices=["all", "spmm", "sddmm", "copy", "mh_sddmm", "mh_spmm", "mh_sddmm_softmax",
+    ap.add_argument("--only", choices=["all", "spmm", "sddmm", "sddmm_shuffled", "copy", "mh_sddmm", "mh_spmm", "mh_sddmm_softmax",
                                        "mh_attention", "mh_attention_kv", "gather_probe", "gather_store_probe"],
                     default="all",
                     help="spmm / sddmm / copy / gather_probe: run just that kernel (for profiler runs), no sweep, no "
@@ -368,8 +368,13 @@ def main():
         spmm = VanillaSpMMhip(adj)
         torch.cuda.synchronize(dev)
         plan_seconds["spmm"] = time.time() - t
-    if args.only in ("all", "sddmm"):
+    if args.only in ("all", "sddmm", "sddmm_shuffled"):
         coo = adj.tocoo()
+        if args.only == "sddmm_shuffled":  # the same edges in a seeded random order (the sweep's shuffled row)
+            import scipy.sparse
+            perm = np.random.default_rng(17).permutation(nnz)
+            coo = scipy.sparse.coo_matrix((coo.data[perm], (coo.row[perm], coo.col[perm])), shape=coo.shape)
+            del perm
         torch.cuda.synchronize(dev)
         t = time.time()
         sddmm = VanillaSDDMMhip(coo)
@@ -387,12 +392,12 @@ def main():
         module.build([placeholder((n_cols, F)), placeholder((n_rows, F))], {}, {})
         return [src, dst]
 
-    if args.only == "sddmm":
+    if args.only in ("sddmm", "sddmm_shuffled"):
         ins = sddmm_case(sddmm, F)
         ms = timed(lambda: sddmm.run(ins), args.steps, args.warmup)
         b = sddmm_alg_bytes(nnz, F)
-        print(json.dumps({"kernel": "sddmm", "F": F, "ms": ms, "alg_GBps": b / ms / 1e6,
-                          "frac": b / ms / 1e6 / HBM_PEAK_GBPS}))
+        print(json.dumps({"kernel": args.only, "F": F, "ms": ms, "alg_GBps": b / ms / 1e6,
+                          "frac": b / ms / 1e6 / HBM_PEAK_GBPS, "plan_seconds": plan_seconds["sddmm"]}))
         return
 
     # ---- the timed step: CSR SpMM, feature length F --------------------------------
