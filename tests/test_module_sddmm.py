@@ -494,3 +494,33 @@ def test_random_structures_under_random_schedules(config_guard, seed):
         out = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
         want = (src[coo.col].astype(np.int64) * dst[coo.row].astype(np.int64)).sum(-1).astype(np.float32)
         assert np.array_equal(out, want), (seed, F)                            # exact on integers
+
+
+def test_plans_give_their_device_memory_back(config_guard):
+    """Plans of every kind (row-sorted list, sorted copy with its routing, re-ordered edge list; SpMM with its
+    re-laid ids) built and destroyed in a loop leave the device's free memory where it was."""
+    import gc
+    import torch
+    from featgraph_amd.module import VanillaSpMMhip
+    _lib.config_set("sddmm.blocked", 1)
+    _lib.config_set("sddmm.block_cols", 500)
+    adj = datasets.config_graph("c2-mini")
+    coo = adj.tocoo()
+    perm = np.random.default_rng(3).permutation(coo.nnz)
+    shuffled = scipy.sparse.coo_matrix((coo.data[perm], (coo.row[perm], coo.col[perm])), shape=coo.shape)
+
+    def cycle():
+        for sorted_copy in (1, 0):
+            _lib.config_set("sddmm.sorted_copy", sorted_copy)
+            for m in (coo, shuffled):
+                VanillaSDDMMhip(m)
+        VanillaSpMMhip(adj)
+        gc.collect()
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
+
+    cycle()                                                          # first use: allocator pools, code objects
+    free0 = torch.cuda.mem_get_info()[0]
+    for _ in range(5):
+        cycle()
+    assert abs(torch.cuda.mem_get_info()[0] - free0) < (8 << 20)    # a plan here holds tens of megabytes
