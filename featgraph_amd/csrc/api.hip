@@ -432,6 +432,7 @@ int *config_slot(const char *key) {
   if (!strcmp(key, "spmm.multi_long")) return &c.spmm_multi_long;
   if (!strcmp(key, "spmm.tile_interleave")) return &c.spmm_tile_interleave;
   if (!strcmp(key, "spmm.relay")) return &c.spmm_relay;
+  if (!strcmp(key, "spmm.general_multi")) return &c.spmm_general_multi;
   if (!strcmp(key, "sddmm.group")) return &c.sddmm_group;
   if (!strcmp(key, "sddmm.batches")) return &c.sddmm_batches;
   if (!strcmp(key, "sddmm.blocked")) return &c.sddmm_blocked;
@@ -630,8 +631,26 @@ int fg_spmm_csr_general_f32(const fg_spmm_plan *plan, const float *feat, const f
   if (plan->nnz > 0 && (!feat || (!vals && msg != FG_MSG_COPY_U)))
     return fg::fail(FG_EINVAL, "feat or edge values are null");
   if (plan->n_rows == 0) return FG_OK;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  // The several-rows-per-wave kernel takes the call where it would take the plain operator (tiles of 32 and 64
+  // floats): same records, same passes, the message and the reducer in place of the multiply-add; the mean is
+  // the sum followed by one division per element.
+  if (plan->nnz > 0 && fg::config().spmm_general_multi != 0) {
+    fg::SpmmArgs a;
+    fg::SpmmShape s;
+    if (int rc = spmm_prepare(plan, feat, vals ? vals : feat, out, 1, F, 0, &a, &s)) return rc;
+    a.reduce = reduce == FG_REDUCE_MEAN ? FG_REDUCE_SUM : reduce;
+    a.msg = msg;
+    const fg::MultiRuns *runs = multi_table(plan, a, 0);
+    if (runs && fg::spmm_multi_general_applies(a)) {
+      if (int rc = multi_run(plan, runs, a, st)) return rc;
+      if (reduce == FG_REDUCE_MEAN)
+        return fg::spmm_mean_finish_launch(plan->indptr, out, static_cast<int32_t>(plan->n_rows), F, st);
+      return FG_OK;
+    }
+  }
   return fg::spmm_general_launch(plan->row_order, plan->seg, plan->n_blocks, plan->indices, vals, feat, out,
-                                 static_cast<int32_t>(plan->n_rows), F, msg, reduce, static_cast<hipStream_t>(stream));
+                                 static_cast<int32_t>(plan->n_rows), F, msg, reduce, st);
 }
 
 int fg_sddmm_coo_general_f32(int64_t nnz, const int32_t *row, const int32_t *col, const float *src, const float *dst,
@@ -944,7 +963,8 @@ int fg_config_set(const char *key, int32_t value) {
                     slot == &fg::config().spmm_buffer_loads || slot == &fg::config().sddmm_fast ||
                     slot == &fg::config().sddmm_buffer_loads || slot == &fg::config().sddmm_rows ||
                     slot == &fg::config().spmm_multi || slot == &fg::config().sddmm_sorted_copy ||
-                    slot == &fg::config().sddmm_regroup || slot == &fg::config().spmm_relay;
+                    slot == &fg::config().sddmm_regroup || slot == &fg::config().spmm_relay ||
+                    slot == &fg::config().spmm_general_multi;
   // flags: 0 / 1 are explicit, anything negative restores the default;
   // sizes: 0 restores the default
   *slot = flag ? (value < 0 ? -1 : (value != 0)) : std::max(value, 0);

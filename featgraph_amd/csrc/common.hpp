@@ -28,7 +28,7 @@ struct Config {
   int spmm_multi = -1, spmm_multi_blocks = 0, spmm_multi_long = 0, spmm_tile_interleave = 0;
   int sddmm_group = 0, sddmm_batches = 0, sddmm_blocked = -1, sddmm_block_cols = 0;
   int sddmm_fast = -1, sddmm_buffer_loads = -1, sddmm_rows = -1, sddmm_rows_blocks = 0;
-  int attention_blocks = 0, sddmm_rows_wide = 0, sddmm_sorted_copy = -1, sddmm_regroup = -1, spmm_relay = -1;
+  int attention_blocks = 0, sddmm_rows_wide = 0, sddmm_sorted_copy = -1, sddmm_regroup = -1, spmm_relay = -1, spmm_general_multi = -1;
 };
 Config &config();
 
@@ -68,6 +68,10 @@ struct SpmmArgs {
   // records over a re-laid copy of the ids (MultiRuns::ids_p): `indices` is that copy, and a run's values start
   // at the CSR position in the record's fourth entry
   int32_t vals_by_csr = 0;
+  // several-rows-per-wave kernel as the generalised operator: reduce = FG_REDUCE_SUM / MAX / MIN folds
+  // msg(feature, value) (FG_MSG_*); reduce < 0 is the plain multiply-add
+  int32_t reduce = -1;
+  int32_t msg = 0;
 };
 
 struct SpmmShape {
@@ -101,6 +105,7 @@ int multi_runs_build(const int32_t *seg, const int32_t *row_order, const int32_t
 void multi_runs_free(MultiRuns *r);
 int spmm_multi_tile(int32_t F);
 bool spmm_multi_applies(const SpmmArgs &a);
+bool spmm_multi_general_applies(const SpmmArgs &a);  // ... with a.reduce >= 0
 int spmm_multi_launch(const SpmmArgs &a, hipStream_t stream);
 
 // One launch of the edge-parallel SDDMM kernel over n_ve = nnz * H dot
@@ -183,6 +188,8 @@ int sddmm_rows_launch(const int32_t *seg, const int32_t *row_order, int32_t n_ro
 int spmm_general_launch(const int32_t *row_order, const int32_t *seg, int32_t n_blocks, const int32_t *indices,
                         const float *vals, const float *feat, float *out, int32_t n_rows, int32_t F, int msg,
                         int reduce, hipStream_t stream);
+// out[r, :] /= degree of row r (rows without nonzeros stay 0): the last step of the mean over a sum
+int spmm_mean_finish_launch(const int32_t *indptr, float *out, int32_t n_rows, int32_t F, hipStream_t stream);
 int sddmm_elementwise_launch(const int32_t *row, const int32_t *col, const float *src, const float *dst, float *out,
                              int64_t nnz, int32_t F, int op, hipStream_t stream);
 

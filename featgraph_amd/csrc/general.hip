@@ -10,6 +10,8 @@
 //          and per fold step (-ffp-contract=off), hence (u*e, sum) equals fg_spmm_csr_f32 bit for bit.
 //   SDDMM  Out[e, f] = Src[col[e], f] op Dst[row[e], f]        op: +, -, *, /   (no reduction over f)
 //
+// The several-rows-per-wave kernel (spmm_multi_kernel.hpp) takes the generalised SpMM where it takes the plain
+// one; the kernel here serves the other shapes.
 // SpMM kernel: rows come in the plan's order (descending degree); a slot of LPR lanes owns one (row, tile)
 // pair, every lane VEC adjacent floats; column ids and values are fetched LPR at a time with one coalesced
 // load, a chunk ahead of their use, and handed out inside the slot with cross-lane reads; sixteen gathers are
@@ -275,6 +277,26 @@ int spmm_general_launch(const int32_t *row_order, const int32_t *seg, int32_t n_
     a.first_pass = b == 0;
     if (int rc = general_pass(a, vec4, msg, reduce, stream)) return rc;
   }
+  return FG_OK;
+}
+
+namespace {
+__global__ __launch_bounds__(kBlockThreads) void mean_finish_kernel(const int32_t *indptr, float *out, int64_t total, int32_t F) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < total; t += stride) {
+    const int64_t r = t / F;
+    const int32_t deg = indptr[r + 1] - indptr[r];
+    if (deg > 0) out[t] = out[t] / static_cast<float>(deg);
+  }
+}
+}  // namespace
+
+int spmm_mean_finish_launch(const int32_t *indptr, float *out, int32_t n_rows, int32_t F, hipStream_t stream) {
+  const int64_t total = static_cast<int64_t>(n_rows) * F;
+  if (total == 0) return FG_OK;
+  const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((total + kBlockThreads - 1) / kBlockThreads, 1 << 16));
+  mean_finish_kernel<<<dim3(blocks), dim3(kBlockThreads), 0, stream>>>(indptr, out, total, F);
+  FG_HIP_TRY(hipGetLastError());
   return FG_OK;
 }
 

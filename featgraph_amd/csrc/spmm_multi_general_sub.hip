@@ -1,0 +1,11 @@
+// The several-rows-per-wave SpMM kernel as the generalised operator with the message FG_MSG_SUB (three reducers, tiles
+// of 32 and 64 floats).
+#include "spmm_multi_kernel.hpp"
+
+namespace fg {
+
+int spmm_multi_general_sub(const SpmmArgs &a, int64_t blocks, hipStream_t stream) {
+  return launch_multi_general<FG_MSG_SUB>(a, blocks, stream);
+}
+
+}  // namespace fg

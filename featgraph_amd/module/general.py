@@ -41,14 +41,21 @@ class GeneralizedSpMMhip(SpMMbase):
 
     def lower_to_ir(self, input_placeholders, compute_args, schedule_args):
         _, H, D, _ = self._parse_build(input_placeholders, compute_args, schedule_args)
-        # the plan's own description tells whether (and into how many) column blocks the matrix is cut
+        # the plan's own description tells which kernel the plain operator would take and whether (and into how
+        # many) column blocks the matrix is cut
         plan_text = super().lower_to_ir(input_placeholders, compute_args, schedule_args)
+        head = "spmm_csr_general rows=%d cols=%d nnz=%d D=%d | msg=%s reduce=%s | " % (
+            self._num_rows, self._num_cols, self._nnz, D, self._msg, self._reduce)
+        # the several-rows-per-wave kernel takes the call where it takes the plain one, for tiles of 32 and 64
+        # floats and feature matrices within 32-bit byte offsets
+        if ("rows-per-wave" in plan_text and D > 16 and self._num_cols * D * 4 < 2 ** 32 and self._num_cols <= 2 ** 24
+                and _lib.config_get("spmm.general_multi") != 0 and _lib.config_get("spmm.buffer_loads") != 0):
+            return head + ("kernel=rows-per-wave with the message and the reducer in place of the multiply-add%s | %s" % (
+                ", then one division per element" if self._reduce == "mean" else "", plan_text.split(" | ")[-1]))
         found = re.search(r"(\d+) column blocks of (\d+)", plan_text)
         passes = ("%s column blocks of %s, one launch per block, the fold carried in the output" % found.groups()
                   if found else "whole rows, 1 launch")
-        return ("spmm_csr_general rows=%d cols=%d nnz=%d D=%d | msg=%s reduce=%s | kernel=row-slot, %s, "
-                "rows=by-descending-degree, tile=64 floats x %d tiles" % (
-                    self._num_rows, self._num_cols, self._nnz, D, self._msg, self._reduce, passes, (D + 63) // 64))
+        return head + "kernel=row-slot, %s, rows=by-descending-degree, tile=64 floats x %d tiles" % (passes, (D + 63) // 64)
 
     def _launch(self, tensors):
         feat = tensors[0]

@@ -130,10 +130,13 @@ FG_API int fg_spmm_csr_noalloc_f32(int64_t n_rows, int64_t n_cols, int64_t nnz, 
  * MEAN is the sum divided by the row's degree (one rounded division).  Rows
  * without nonzeros give 0 under every reducer.  One rounded operation per
  * message and per fold step, so (MUL, SUM) equals fg_spmm_csr_f32 bit for bit.
- * vals may be null for FG_MSG_COPY_U.  One launch per column block of the
- * plan (one launch over whole rows when the plan has no blocks); the partial
- * fold of a row is carried in `out` between launches, so `out` must not be
- * read by anything else on the stream until the last launch has finished.
+ * vals may be null for FG_MSG_COPY_U.  Runs the kernel of fg_spmm_csr_f32 with
+ * the message and the reducer in place of the multiply-add where that kernel
+ * applies (feature lengths that are multiples of 4 above 16), a row-slot kernel
+ * otherwise; one launch per column block of the plan (one launch over whole
+ * rows when the plan has no blocks), MEAN one more for the division.  The
+ * partial fold of a row is carried in `out` between launches, so `out` must
+ * not be read by anything else on the stream until the last launch has finished.
  */
 #define FG_MSG_MUL 0
 #define FG_MSG_ADD 1
@@ -361,7 +364,8 @@ FG_API int64_t fg_probe_store_rows_f32(float *out, int64_t n_out_rows, int32_t r
  * "spmm.multi_long" (run length from which a run gets a wave of its own,
  * default 512; read at plan creation), "spmm.tile_interleave" (feature tiles
  * whose workgroups alternate inside one launch of that kernel: 1 or 2, default 2),
- * "spmm.relay" (0/1: whether the plan keeps, per pass layout of that kernel, a
+ * "spmm.general_multi" (0/1: whether fg_spmm_csr_general_f32 may use that
+ * kernel; default 1), "spmm.relay" (0/1: whether the plan keeps, per pass layout of that kernel, a
  * copy of the column ids in the order the passes visit them; read at plan
  * creation; default 1),
  * "sddmm.blocked" (0/1: never / always build and use column blocks, read at

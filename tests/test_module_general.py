@@ -69,24 +69,30 @@ def test_column_block_passes_fold_in_the_same_order(msg, reduce):
     adj = adj.tocsr()
     adj.sort_indices()
     adj.data = (adj.data + np.float32(0.25)).astype(np.float32)
-    feat = datasets.spmm_operands(adj, 72)                # a whole tile and a partial one
-    feat[adj.indices[adj.indptr[7]]] = np.nan             # first message of row 7 (and wherever else the vertex occurs)
-    feat[adj.indices[adj.indptr[9] + 3]] = np.nan         # a later message of row 9
-    want = ref.spmm_general(adj.indptr, adj.indices, adj.data, feat, msg, reduce)
     try:
         _lib.config_set("spmm.blocked", 1)
-        for block_cols in (64, 1500):
-            _lib.config_set("spmm.block_cols", block_cols)
-            module = GeneralizedSpMMhip(adj, msg, reduce)
-            assert "column blocks" in module.lower_to_ir([placeholder(feat.shape)], {}, {})
-            module.build([placeholder(feat.shape)], {}, {})
-            module.out_tvm.tensor.fill_(7.0)
-            out = module.run([nd.array(feat, module.ctx)]).asnumpy()
-            assert np.array_equal(out, want, equal_nan=True), block_cols
-            assert not out[5].any() and not out[4242].any()
+        # 72 floats: a whole 64-float tile and a partial one; 24: one partial 32-float tile.  Both kernels: the
+        # several-rows-per-wave one (also one wave per run of 512 nonzeros and more) and the row-slot one.
+        for F, multi in ((72, -1), (72, 0), (24, -1)):
+            feat = datasets.spmm_operands(adj, F)
+            feat[adj.indices[adj.indptr[7]]] = np.nan         # first message of row 7 (and wherever else the vertex occurs)
+            feat[adj.indices[adj.indptr[9] + 3]] = np.nan     # a later message of row 9
+            want = ref.spmm_general(adj.indptr, adj.indices, adj.data, feat, msg, reduce)
+            _lib.config_set("spmm.general_multi", multi)
+            for block_cols in (64, 1500):
+                _lib.config_set("spmm.block_cols", block_cols)
+                module = GeneralizedSpMMhip(adj, msg, reduce)
+                text = module.lower_to_ir([placeholder(feat.shape)], {}, {})
+                assert "column blocks" in text and ("rows-per-wave" in text) == (multi != 0)
+                module.build([placeholder(feat.shape)], {}, {})
+                module.out_tvm.tensor.fill_(7.0)
+                out = module.run([nd.array(feat, module.ctx)]).asnumpy()
+                assert np.array_equal(out, want, equal_nan=True), (F, multi, block_cols)
+                assert not out[5].any() and not out[4242].any()
     finally:
         _lib.config_set("spmm.blocked", -1)
         _lib.config_set("spmm.block_cols", 0)
+        _lib.config_set("spmm.general_multi", -1)
 
 
 def test_mul_sum_is_the_vanilla_kernel_and_max_min_match_numpy(adj_127x255):
