@@ -141,7 +141,7 @@ struct SddmmBlocks {
   int32_t block_cols = 0;
 };
 
-// Copy of a COO edge list sorted by (row, column) (sddmm_blocked.hip): lets the row-run kernel serve a list in
+// Copy of a COO edge list sorted by (row, column) (sddmm_sorted.hip): lets the row-run kernel serve a list in
 // any order.  Device arrays owned by the SDDMM plan, all null when there is no such copy.
 struct SddmmSorted {
   int32_t *row_s = nullptr;    // [nnz] row ids in sorted order; freed once the row pointer is built
