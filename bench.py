@@ -91,6 +91,16 @@ def committed_traffic(op, graph, F):
     return (float(m.group(1)), rel) if m else (None, None)
 
 
+def committed_hit_rate(op, graph, F):
+    """(L2 hit rate of the operator's kernels as a fraction, source file) from the same summary, or (None, None)."""
+    rel = os.path.join("profiles", "%s_%s_counters.txt" % (op, graph))
+    path = os.path.join(ROOT, rel)
+    if not os.path.exists(path):
+        return None, None
+    m = re.search(r"^feat-len %d .*?L2 hit rate ([0-9.]+) %%" % F, open(path).read(), flags=re.M | re.S)
+    return (float(m.group(1)) / 100.0, rel) if m else (None, None)
+
+
 def committed_traffic_mh(kind, D):
     """The same for a multi-head operator on the 2.45M-vertex graph."""
     rel = os.path.join("profiles", "multihead_c4_counters.txt")
@@ -128,6 +138,8 @@ def main():
                     help="spmm / sddmm / copy / gather_probe: run just that kernel (for profiler runs), no sweep, no "
                          "CPU leg; mh_sddmm / mh_spmm: the multi-head operators (8 heads of --feat-len floats, use "
                          "--graph c4)")
+    ap.add_argument("--band-rows", type=int, default=0,
+                    help="with --only gather_probe: rows per band (default 16384 rows of a 64-float tile)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg and the parity checks")
     ap.add_argument("--no-sweep", action="store_true", help="skip the feature-length sweep")
     ap.add_argument("--no-mh", action="store_true", help="skip the multi-head operators on the 2.45M-vertex graph")
@@ -167,19 +179,34 @@ def main():
 
     sink = torch.zeros(64, dtype=torch.float32, device=dev)
 
-    def gather_probe(feat_t, n_gathers, steps=5, warmup=3):
-        """Milliseconds that the bare gather pattern takes for n_gathers row gathers per tile, with the tile width and
-        band width of the operators (a 4 MB band: 16384 rows of a 64-float tile)."""
+    def gather_probe(feat_t, n_gathers, steps=5, warmup=3, band=None):
+        """Milliseconds that the bare gather pattern takes for n_gathers row gathers per tile, with the tile width of
+        the operators and a band of `band` rows (default: a 4 MB band, 16384 rows of a 64-float tile, which an L2
+        holds: nearly every gather hits)."""
         n, F = feat_t.shape
         tile = 64 if F >= 64 else (32 if F >= 32 else 16)
         if F % tile != 0 or n * F * 4 >= 2 ** 32:
             return None
-        band = 16384 * (64 // tile)
+        band = int(band) if band else 16384 * (64 // tile)
         issued = L.fg_probe_gather_count(n, tile, band, n_gathers)
         ms = timed(lambda: _lib.check(L.fg_probe_gather_f32(feat_t.data_ptr(), n, F, tile, band, n_gathers,
                                                             sink.data_ptr(), stream.cuda_stream)), steps, warmup)
         return {"ms": ms * n_gathers / issued, "tile": tile, "band_rows": band, "gathers_per_tile": n_gathers,
                 "row_TBps": n_gathers * F * 4 / (ms * n_gathers / issued) / 1e9}
+
+    def gather_probe_at_hit_rate(feat_t, n_gathers, op, F):
+        """The same probe with its band widened until its own L2 hit rate is the operator's: gathers that fall
+        uniformly on a band of b L2 sizes hit at 1 / b (measured: profiles/gather_probe_c2_f64_bands.txt), so the
+        band is 16384 / hit_rate rows of a 64-float tile.  What the memory system does for this gather stream at
+        the hit rate the operator reaches, with no ids, values, sums or results beside it."""
+        hit, src_file = committed_hit_rate(op, args.graph, F)
+        if not hit:
+            return None
+        tile = 64 if F >= 64 else (32 if F >= 32 else 16)
+        p = gather_probe(feat_t, n_gathers, band=min(feat_t.shape[0], round(16384 * (64 // tile) / hit)))
+        if p:
+            p.update({"l2_hit_rate_of_the_operator": hit, "hit_rate_source": src_file})
+        return p
 
     def rows_probe(feat_t, n_gathers, steps=3):
         """Milliseconds that n_gathers random whole-row gathers from feat_t take (rows of 128 .. 1024 floats)."""
@@ -230,7 +257,7 @@ def main():
 
     if args.only == "gather_probe":
         feat_t = device_normal((n_cols, F), 1)
-        p = gather_probe(feat_t, nnz, args.steps)
+        p = gather_probe(feat_t, nnz, args.steps, band=args.band_rows or None)
         print(json.dumps({"kernel": "gather_probe", "F": F, **(p or {})}))
         return
 
@@ -411,6 +438,7 @@ def main():
     gpu_out = spmm.out_tvm.asnumpy() if args.only == "all" else None
     traffic, traffic_source = committed_traffic("spmm", args.graph, F)
     probe = gather_probe(feat.tensor, nnz) if args.only == "all" else None
+    probe_hit = gather_probe_at_hit_rate(feat.tensor, nnz, "spmm", F) if args.only == "all" else None
     roofline = {
         "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
         "traffic": traffic, "traffic_source": traffic_source,
@@ -418,9 +446,13 @@ def main():
         "compulsory_bytes": b_min, "hbm_frac_compulsory": b_min / ms / 1e6 / HBM_PEAK_GBPS,
         "l2_fabric_frac": (traffic / ms / 1e6 / HBM_PEAK_GBPS) if traffic else None,
         "gather_ceiling": probe, "frac_of_gather_ceiling": (probe["ms"] / ms) if probe else None,
+        "gather_at_the_operators_l2_hit_rate": probe_hit,
+        "frac_of_gather_at_the_operators_l2_hit_rate": (probe_hit["ms"] / ms) if probe_hit else None,
         "note": "`achieved` is the gather model (no cache reuse credited): most of those bytes are served by L2 / "
                 "Infinity Cache and never reach HBM, so `frac` is not bounded by 1 on this graph; "
-                "hbm_frac_compulsory, l2_fabric_frac and frac_of_gather_ceiling are. One operator launch is one "
+                "hbm_frac_compulsory, l2_fabric_frac and the two frac_of_gather_* are (the bare gather stream with "
+                "nearly every gather hitting L2, and with the band widened until the probe's hit rate is the "
+                "operator's). One operator launch is one "
                 "dispatch per column-block pass and feature tile (see `launch`); bytes, time and traffic are per "
                 "operator launch. `traffic` is read from the committed profile named in traffic_source, not "
                 "measured in this run."}
@@ -477,12 +509,16 @@ def main():
             b = spmm_alg_bytes(nnz, n_rows, f)
             tr, src_file = committed_traffic("spmm", args.graph, f)
             p = gather_probe(x.tensor, nnz)
+            ph = gather_probe_at_hit_rate(x.tensor, nnz, "spmm", f)
+            ph_sddmm = gather_probe_at_hit_rate(x.tensor, nnz, "sddmm", f)  # same gathers, SDDMM's hit rate
             row = {"op": "spmm", "F": f, "ms": sec * 1e3, "GFLOPs": 2.0 * nnz * f / sec / 1e9,
                    "alg_GBps": b / sec / 1e9, "frac": b / sec / 1e9 / HBM_PEAK_GBPS,
                    "hbm_frac_compulsory": spmm_min_bytes(nnz, n_rows, n_cols, f) / sec / 1e9 / HBM_PEAK_GBPS,
                    "traffic": tr, "traffic_source": src_file,
                    "gather_ceiling_ms": p["ms"] if p else None,
-                   "frac_of_gather_ceiling": p["ms"] / (sec * 1e3) if p else None}
+                   "frac_of_gather_ceiling": p["ms"] / (sec * 1e3) if p else None,
+                   "gather_at_the_operators_l2_hit_rate": ph,
+                   "frac_of_gather_at_the_operators_l2_hit_rate": ph["ms"] / (sec * 1e3) if ph else None}
             if check:
                 t0 = time.time()
                 want = ref.spmm_csr_x86(adj.indptr, adj.indices, adj.data, x.tensor.cpu().numpy())
@@ -501,7 +537,9 @@ def main():
                    "hbm_frac_compulsory": sddmm_min_bytes(nnz, n_rows, n_cols, f) / sec / 1e9 / HBM_PEAK_GBPS,
                    "traffic": tr, "traffic_source": src_file,
                    "gather_ceiling_ms": p["ms"] if p else None,
-                   "frac_of_gather_ceiling": p["ms"] / (sec * 1e3) if p else None}
+                   "frac_of_gather_ceiling": p["ms"] / (sec * 1e3) if p else None,
+                   "gather_at_the_operators_l2_hit_rate": ph_sddmm,
+                   "frac_of_gather_at_the_operators_l2_hit_rate": ph_sddmm["ms"] / (sec * 1e3) if ph_sddmm else None}
             if check:
                 out = sddmm.out_tvm.asnumpy()
                 s_h, d_h = ins[0].tensor.cpu().numpy(), ins[1].tensor.cpu().numpy()
