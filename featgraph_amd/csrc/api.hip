@@ -46,6 +46,7 @@ struct fg_spmm_plan {
   // n_blocks > 1 only when every row's column ids ascend.
   int32_t *seg;  // owned, device, (n_blocks + 1) * n_rows entries
   int32_t n_blocks;
+  bool cols_unsorted = false;  // blocks were wanted but some row's column ids descend
   int32_t block_cols;
   // When the library sizes the blocks it may cut each block of the default width into `split` equal ones, so
   // that a kernel can take 1 .. split neighbouring blocks per pass; split_used is 1 when the caller sized them.
@@ -78,6 +79,7 @@ struct fg_sddmm_plan {
   // Any other list with valid ids: a copy sorted by (row, column), over which `indptr` and `rows` are then
   // built; the row-run kernel writes its results in that order and a gather returns them to the caller's.
   fg::SddmmSorted sorted;
+  bool input_row_sorted = false;  // the caller's own list has ascending row ids (indptr then describes it too)
 };
 
 static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr, const int32_t *indices,
@@ -404,6 +406,7 @@ int build_bounds(fg_spmm_plan *p) {
     if (unsorted && n_blocks > 1) {  // blocks would reorder the sums of such rows
       (void)hipFree(seg);
       n_blocks = 1;
+      p->cols_unsorted = true;
       continue;
     }
     p->seg = seg;
@@ -729,6 +732,28 @@ static int build_row_runs(fg_sddmm_plan *p, int32_t num_col_partitions) {
     p->indptr = nullptr;
     fg::sddmm_sorted_free(&p->sorted);
   }
+  p->input_row_sorted = !bad;
+  if (!bad && p->rows && p->rows->cols_unsorted && fg::config().sddmm_sorted_copy != 0) {
+    // Rows ascend but the columns inside some row do not, so the rows could not be cut into column blocks: a
+    // copy sorted inside the rows can.  The row pointer is the same for both, and so is the visiting order.
+    if (int rc = fg::sddmm_sorted_build(p->nnz, p->n_rows, p->n_cols, p->row, p->col, &p->sorted)) return rc;
+    if (p->sorted.col_s) {
+      (void)hipFree(p->sorted.row_s);
+      p->sorted.row_s = nullptr;
+      fg_spmm_plan *blocked = nullptr;
+      if (int rc = row_plan_create(p->n_rows, p->n_cols, p->nnz, p->indptr, p->sorted.col_s, num_col_partitions,
+                                   fg::config().sddmm_block_cols, kSddmmBlockCols, kSddmmSplit,
+                                   fg::config().sddmm_blocked, 8.0, false, &blocked))
+        return rc;
+      if (blocked && blocked->seg && blocked->n_blocks >= 2) {
+        fg_spmm_plan_destroy(p->rows);
+        p->rows = blocked;
+      } else {
+        if (blocked) fg_spmm_plan_destroy(blocked);
+        fg::sddmm_sorted_free(&p->sorted);
+      }
+    }
+  }
   return FG_OK;
 }
 
@@ -872,7 +897,7 @@ int fg_sddmm_softmax_plan_f32(const fg_sddmm_plan *plan, const float *src, const
   if (plan->nnz == 0) return FG_OK;
   if (int rc = check_device(plan->device)) return rc;
   if (!src || !dst || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
-  if (!plan->indptr || !plan->rows || plan->sorted.col_s)
+  if (!plan->indptr || !plan->rows || !plan->input_row_sorted)
     return fg::fail(FG_EUNSUPPORTED, "edge softmax needs a row-sorted edge list (each destination row's edges consecutive)");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int32_t n = static_cast<int32_t>(plan->n_rows);

@@ -200,9 +200,11 @@ FG_API int fg_sddmm_coo_general_f32(int64_t nnz, const int32_t *row, const int32
  * results, so they are always written in the caller's edge order (there is no
  * edge_mapping to apply) and equal the sorted list's bit for bit.  Because the results pass through memory that the plan
  * owns, two calls on ONE plan of an unsorted list must not overlap in time.
- * Rows that ascend while their columns do not, lists with ids outside the
- * matrix and "sddmm.sorted_copy" = 0 fall back to a copy re-ordered by column
- * block and destination row whose kernel scatters its results.
+ * A list whose rows ascend while the columns inside a row do not gets the same
+ * sorted copy (and may still be used with fg_sddmm_softmax_plan_f32, which
+ * works on the caller's order).  Lists with ids outside the matrix and
+ * "sddmm.sorted_copy" = 0 fall back to a copy re-ordered by column block and
+ * destination row whose kernel scatters its results.
  * The plan BORROWS row and col, which must stay alive and unchanged until
  * fg_sddmm_plan_destroy.
  */

@@ -298,7 +298,10 @@ def test_which_lists_take_the_row_run_kernel(config_guard):
     order = np.lexsort((rng.random(coo.nnz), coo.row))
     ragged = scipy.sparse.coo_matrix((coo.data[order], (coo.row[order], coo.col[order])), shape=coo.shape)
     assert np.all(np.diff(ragged.row) >= 0) and np.any(np.diff(ragged.col)[np.diff(ragged.row) == 0] < 0)
+    assert "sorted by row and column" in _describe(VanillaSDDMMhip(ragged), src, dst)
+    _lib.config_set("sddmm.sorted_copy", 0)
     assert "column-blocked edge list" in _describe(VanillaSDDMMhip(ragged), src, dst)
+    _lib.config_set("sddmm.sorted_copy", -1)
     base = _run_sddmm(coo, src, dst)
     inv = np.empty_like(order)
     inv[order] = np.arange(coo.nnz)

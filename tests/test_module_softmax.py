@@ -108,3 +108,26 @@ def test_fused_operator_rejects_an_unsorted_edge_list():
     shuffled = scipy.sparse.coo_matrix((adj.data[perm], (adj.row[perm], adj.col[perm])), shape=adj.shape)
     with pytest.raises(ValueError):
         MultiHeadSDDMMSoftmaxhip(shuffled)
+
+
+@pytest.mark.parametrize("H,D", [(8, 16), (1, 64)])
+def test_fused_operator_on_rows_whose_columns_do_not_ascend(H, D):
+    """Rows ascend, the columns inside a row come in any order: the plan of such a list holds a copy sorted inside
+    the rows for the single-head row-run kernel, while the softmax still runs over the caller's own order."""
+    adj = datasets.config_graph("c2-mini")
+    coo = adj.tocoo()
+    rng = np.random.default_rng(7)
+    order = np.lexsort((rng.random(coo.nnz), coo.row))
+    ragged = scipy.sparse.coo_matrix((coo.data[order], (coo.row[order], coo.col[order])), shape=coo.shape)
+    src, dst = datasets.sddmm_operands(coo, (H, D))
+    src *= np.float32(0.25)
+    try:
+        _lib.config_set("sddmm.blocked", 1)
+        _lib.config_set("sddmm.block_cols", 500)
+        out, _ = _fused(ragged, src, dst)
+    finally:
+        _lib.config_set("sddmm.blocked", -1)
+        _lib.config_set("sddmm.block_cols", 0)
+    scores64 = np.einsum("ehd,ehd->eh", src[ragged.col].astype(np.float64), dst[ragged.row].astype(np.float64))
+    want = ref.edge_softmax(adj.indptr, scores64.astype(np.float32))
+    np.testing.assert_allclose(out, want, rtol=5e-5, atol=1e-7)
