@@ -30,6 +30,7 @@ SIGNATURES = {
     "fg_sddmm_plan_create_partitioned": (ctypes.c_int, [_i64, _i64, _i64, _p, _p, _i32, ctypes.POINTER(_p)]),
     "fg_sddmm_plan_destroy": (None, [_p]),
     "fg_sddmm_coo_plan_f32": (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _p]),
+    "fg_sddmm_coo_general_plan_f32": (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _p]),
     "fg_edge_softmax_csr_f32": (ctypes.c_int, [_i64, _p, _p, _p, _i32, _p]),
     "fg_sddmm_softmax_plan_f32": (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _p]),
     "fg_attention_csr_mh_f32": (ctypes.c_int, [_p, _p, _p, _p, _p, _i32, _i32, _p]),

@@ -881,6 +881,28 @@ int fg_sddmm_coo_plan_f32(const fg_sddmm_plan *plan, const float *src, const flo
                                   plan->n_rows * int64_t{D} * 4, static_cast<hipStream_t>(stream));
 }
 
+int fg_sddmm_coo_general_plan_f32(const fg_sddmm_plan *plan, const float *src, const float *dst, float *out, int32_t F,
+                                  int32_t edge_op, void *stream) {
+  if (!plan) return fg::fail(FG_EINVAL, "plan is null");
+  if (edge_op == FG_EDGE_DOT) return fg_sddmm_coo_plan_f32(plan, src, dst, out, 1, F, stream);
+  if (edge_op < FG_EDGE_DOT || edge_op > FG_EDGE_DIV)
+    return fg::fail(FG_EINVAL, "edge_op = %d is not an FG_EDGE_* code", edge_op);
+  if (int rc = check_heads(1, F)) return rc;
+  if (plan->nnz == 0) return FG_OK;
+  if (int rc = check_device(plan->device)) return rc;
+  if (!src || !dst || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  // the row-run schedule for the caller's own row-sorted list (a sorted copy would leave the [nnz, F] result in
+  // the copy's order); everything else takes the edge-parallel kernel
+  const fg_spmm_plan *r = plan->rows;
+  if (r && r->seg && r->n_blocks >= 2 && !plan->sorted.col_s && fg::config().sddmm_rows != 0 && F % 4 == 0 &&
+      fg::aligned_to(src, 16) && fg::aligned_to(dst, 16) && fg::aligned_to(out, 16))
+    return fg::sddmm_rows_elementwise_launch(r->seg, r->row_order, static_cast<int32_t>(r->n_rows), r->n_blocks,
+                                             std::max(1, sddmm_rows_merge64(plan)), plan->col, src, dst, out,
+                                             plan->n_cols * int64_t{F} * 4, plan->n_rows * int64_t{F} * 4, F, edge_op, st);
+  return fg::sddmm_elementwise_launch(plan->row, plan->col, src, dst, out, plan->nnz, F, edge_op, st);
+}
+
 int fg_edge_softmax_csr_f32(int64_t n_rows, const int32_t *indptr, const float *scores, float *out, int32_t H,
                             void *stream) {
   if (n_rows < 0 || n_rows >= 0x7fffffffLL) return fg::fail(FG_EINVAL, "n_rows = %lld is out of range", (long long)n_rows);

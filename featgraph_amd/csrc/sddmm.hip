@@ -387,6 +387,118 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_rows_kernel(const RowsArg
   }
 }
 
+// The row-run schedule for the elementwise edge functions, Out[e, :] = Src[col[e], :] op Dst[row[e], :]: the same
+// (column block, row) work items, the row's Dst tile in registers, one gathered Src tile per edge out of a band
+// that an L2 holds -- and a 16-byte store per lane in place of the reduction, the edges of a round next to each
+// other in Out.  The edge-parallel kernel of general.hip gathers both rows from all over the matrices; on the
+// 114.6M-edge benchmark graph its Src gathers cross the L2 boundary once per edge, as much traffic again as the
+// result itself.
+template <int OP, bool BUF, int G>
+__global__ __launch_bounds__(kBlockThreads) void sddmm_rows_elementwise_kernel(const RowsArgs a) {
+  constexpr int NG = kWaveSize / G;  // edges per round
+  constexpr int R = 4;               // rounds whose gathers are issued together; two such batches alternate
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int gl = lane & (G - 1);
+  const int g = lane / G;
+  const int n_waves = gridDim.x * kWavesPerBlock;
+  const int n = a.n_rows;
+  int item = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)));
+  const int32_t *const seg_lo = a.seg + static_cast<int64_t>(blockIdx.y) * a.merge * n;
+  const int32_t *const seg_hi = a.seg + static_cast<int64_t>(min((blockIdx.y + 1) * a.merge, a.n_blocks)) * n;
+  const VertexRows<BUF> src(a.src, a.src_bytes), dst(a.dst, a.dst_bytes);
+  const uint32_t row_bytes = static_cast<uint32_t>(a.F) * 4u;
+  const bool kok = gl * 4 < a.valid;  // lanes past the tile's end re-read its last four floats and store nothing
+  const uint32_t lane_bytes = static_cast<uint32_t>(a.first + (kok ? gl * 4 : a.valid - 4)) * 4u;
+  float *const out_lane = a.out + a.first + gl * 4;
+  const int64_t F = a.F;
+
+  auto bounds = [&](int it, int &lo, int &hi, int &row) {
+    lo = hi = row = 0;
+    if (it < n) {
+      lo = seg_lo[it];
+      hi = seg_hi[it];
+      row = a.row_order[it];
+    }
+  };
+  auto first_block = [&](int lo, int hi, int row, int &col, float4 &y) {
+    col = 0;
+    y = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (hi > lo) {
+      if (lane < hi - lo) col = a.col[lo + lane];
+      y = dst.load(row, row_bytes, lane_bytes);
+    }
+  };
+
+  int lo_a, hi_a, row_a, col_a, lo_b, hi_b, row_b;
+  float4 y_a;
+  bounds(item, lo_a, hi_a, row_a);
+  first_block(lo_a, hi_a, row_a, col_a, y_a);
+  bounds(item + n_waves, lo_b, hi_b, row_b);
+
+  while (item < n) {
+    int lo_c, hi_c, row_c, col_b = 0;
+    float4 y_b = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    bounds(item + 2 * n_waves, lo_c, hi_c, row_c);
+    bool next_asked = false;
+    auto ask_next = [&]() {
+      if (!next_asked) first_block(lo_b, hi_b, row_b, col_b, y_b);
+      next_asked = true;
+    };
+
+    for (int e = lo_a; e < hi_a; e += kWaveSize) {
+      const int cnt = min(kWaveSize, hi_a - e);
+      int col_n = 0;
+      const int rounds = (cnt + NG - 1) / NG;
+      float4 xa[R], xb[R];
+      auto issue = [&](int rb, float4(&x)[R]) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          // edges past the run's end read column id 0 of an idle lane: a valid row, nothing stored
+          const int cc = __builtin_amdgcn_ds_bpermute(((NG * (rb + r) + g) & 63) << 2, col_a);
+          x[r] = src.load(cc, row_bytes, lane_bytes);
+        }
+      };
+      auto store = [&](int rb, const float4(&x)[R]) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const int idx = NG * (rb + r) + g;
+          float4 v;
+          if constexpr (OP == FG_EDGE_ADD) v = make_float4(x[r].x + y_a.x, x[r].y + y_a.y, x[r].z + y_a.z, x[r].w + y_a.w);
+          if constexpr (OP == FG_EDGE_SUB) v = make_float4(x[r].x - y_a.x, x[r].y - y_a.y, x[r].z - y_a.z, x[r].w - y_a.w);
+          if constexpr (OP == FG_EDGE_MUL) v = make_float4(x[r].x * y_a.x, x[r].y * y_a.y, x[r].z * y_a.z, x[r].w * y_a.w);
+          if constexpr (OP == FG_EDGE_DIV) v = make_float4(x[r].x / y_a.x, x[r].y / y_a.y, x[r].z / y_a.z, x[r].w / y_a.w);
+          if (idx < cnt && kok) *reinterpret_cast<float4 *>(out_lane + static_cast<int64_t>(e + idx) * F) = v;
+        }
+      };
+      issue(0, xa);
+      {  // behind this run's first gathers: the next run's operands and this run's next 64 ids
+        ask_next();
+        const int more = hi_a - (e + kWaveSize);
+        if (lane < more) col_n = a.col[e + kWaveSize + lane];
+      }
+      for (int rb = 0; rb < rounds; rb += 2 * R) {
+        const bool second = rb + R < rounds;
+        if (second) issue(rb + R, xb);
+        store(rb, xa);
+        if (rb + 2 * R < rounds) issue(rb + 2 * R, xa);
+        if (second) store(rb + R, xb);
+      }
+      col_a = col_n;
+    }
+    ask_next();
+
+    lo_a = lo_b;
+    hi_a = hi_b;
+    row_a = row_b;
+    col_a = col_b;
+    y_a = y_b;
+    lo_b = lo_c;
+    hi_b = hi_c;
+    row_b = row_c;
+    item += n_waves;
+  }
+}
+
 template <int VEC, int G>
 int launch(const SddmmArgs &a, hipStream_t stream) {
   const int64_t per_wave = static_cast<int64_t>(a.batches) * kWaveSize;
@@ -547,6 +659,60 @@ int sddmm_rows_launch(const int32_t *seg, const int32_t *row_order, int32_t n_ro
       rows_dispatch<16, 1>(a, acc, buf, grid, stream);
     else
       rows_dispatch<16, 2>(a, acc, buf, grid, stream);
+    FG_HIP_TRY(hipGetLastError());
+    first += a.valid;
+  }
+  return FG_OK;
+}
+
+template <int OP>
+static void rows_elementwise_dispatch(const RowsArgs &a, int tile, bool buf, dim3 grid, hipStream_t stream) {
+  if (tile == 16) {
+    if (buf) sddmm_rows_elementwise_kernel<OP, true, 4><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+    else sddmm_rows_elementwise_kernel<OP, false, 4><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+  } else if (tile == 32) {
+    if (buf) sddmm_rows_elementwise_kernel<OP, true, 8><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+    else sddmm_rows_elementwise_kernel<OP, false, 8><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+  } else {
+    if (buf) sddmm_rows_elementwise_kernel<OP, true, 16><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+    else sddmm_rows_elementwise_kernel<OP, false, 16><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+  }
+}
+
+// Out [nnz, F]; same tables and pass widths as sddmm_rows_launch, one launch per tile of 16 / 32 / 64 floats,
+// each writing its slice of every edge's row.  src / dst / out 16-byte aligned, F a multiple of 4.
+int sddmm_rows_elementwise_launch(const int32_t *seg, const int32_t *row_order, int32_t n_rows, int32_t n_blocks,
+                                  int32_t merge64, const int32_t *col, const float *src, const float *dst, float *out,
+                                  int64_t src_bytes, int64_t dst_bytes, int32_t F, int op, hipStream_t stream) {
+  if (n_rows == 0) return FG_OK;
+  if (op < FG_EDGE_ADD || op > FG_EDGE_DIV) return fail(FG_EINVAL, "edge_op = %d is not an elementwise FG_EDGE_* code", op);
+  RowsArgs a;
+  a.seg = seg;
+  a.row_order = row_order;
+  a.col = col;
+  a.src = src;
+  a.dst = dst;
+  a.out = out;
+  a.src_bytes = src_bytes;
+  a.dst_bytes = dst_bytes;
+  a.n_rows = n_rows;
+  a.F = F;
+  int64_t blocks = config().sddmm_rows_blocks > 0 ? config().sddmm_rows_blocks : 16384;
+  blocks = std::max<int64_t>(1, std::min<int64_t>(blocks, (n_rows + kWavesPerBlock - 1) / kWavesPerBlock));
+  a.n_blocks = n_blocks;
+  const bool buf = src_bytes < (int64_t{1} << 32) && dst_bytes < (int64_t{1} << 32) && config().sddmm_buffer_loads != 0;
+  for (int first = 0; first < F;) {
+    const int tile = sddmm_rows_tile(F - first, 1);
+    a.merge = std::max(1, std::min(merge64 * (64 / tile), n_blocks));
+    a.first = first;
+    a.valid = std::min(F - first, tile);
+    const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>((n_blocks + a.merge - 1) / a.merge));
+    switch (op) {
+      case FG_EDGE_ADD: rows_elementwise_dispatch<FG_EDGE_ADD>(a, tile, buf, grid, stream); break;
+      case FG_EDGE_SUB: rows_elementwise_dispatch<FG_EDGE_SUB>(a, tile, buf, grid, stream); break;
+      case FG_EDGE_MUL: rows_elementwise_dispatch<FG_EDGE_MUL>(a, tile, buf, grid, stream); break;
+      default: rows_elementwise_dispatch<FG_EDGE_DIV>(a, tile, buf, grid, stream); break;
+    }
     FG_HIP_TRY(hipGetLastError());
     first += a.valid;
   }

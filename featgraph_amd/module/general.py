@@ -88,6 +88,13 @@ class GeneralizedSDDMMhip(SDDMMbase):
         if self._op == "dot":
             return super().lower_to_ir(input_placeholders, compute_args, schedule_args)
         _, _, D = self._parse_build(input_placeholders, compute_args, schedule_args)
+        # the elementwise operators share the dot product's row-run schedule when the plan has one for the
+        # caller's own list (a sorted copy would leave the [nnz, D] result in the copy's order)
+        plan_text = super().lower_to_ir(input_placeholders, compute_args, schedule_args)
+        if "row runs (row-sorted edge list)" in plan_text and D % 4 == 0:
+            found = re.search(r"(\d+) column blocks of (\d+)", plan_text)
+            return ("sddmm_coo_general nnz=%d D=%d | op=%s | kernel=row runs, Dst tile in registers, one store per "
+                    "gathered Src tile, %s column blocks" % (self._nnz, D, self._op, found.group(1) if found else "?"))
         return "sddmm_coo_general nnz=%d D=%d | op=%s | kernel=thread per (edge, 4 floats), 1 launch" % (
             self._nnz, D, self._op)
 
@@ -95,9 +102,9 @@ class GeneralizedSDDMMhip(SDDMMbase):
         if self._op == "dot":
             return super()._launch(tensors)
         src, dst = tensors
-        _lib.check(_lib.lib().fg_sddmm_coo_general_f32(
-            self._nnz, self._adj_row_dev.data_ptr(), self._adj_col_dev.data_ptr(), src.data_ptr(), dst.data_ptr(),
-            self.out_tvm.tensor.data_ptr(), self._D, EDGE_OPS[self._op], C.current_stream_handle(self._ctx)))
+        _lib.check(_lib.lib().fg_sddmm_coo_general_plan_f32(
+            self._plan, src.data_ptr(), dst.data_ptr(), self.out_tvm.tensor.data_ptr(), self._D, EDGE_OPS[self._op],
+            C.current_stream_handle(self._ctx)))
 
 
 class VanillaSpMMGradhip:

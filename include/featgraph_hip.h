@@ -231,6 +231,18 @@ FG_API int fg_sddmm_coo_plan_f32(const fg_sddmm_plan *plan, const float *src, co
 FG_API int fg_sddmm_plan_describe(const fg_sddmm_plan *plan, int32_t H, int32_t D, char *buf, int64_t cap);
 
 /*
+ * fg_sddmm_coo_general_f32 on the plan's edge list (the edgefunc slot of
+ * op/vanilla_sddmm.py:43-47 behind the plan that SDDMMbase.__init__ builds).
+ * For a row-sorted list with column blocks the elementwise operators run over
+ * the plan's (row, column block) runs, the Dst tile held in registers and the
+ * Src gathers inside a band an L2 holds; other lists take the edge-parallel
+ * kernel.  out [nnz, F] (FG_EDGE_DOT: [nnz]); every element is one rounded
+ * operation, so both kernels give the same bits.
+ */
+FG_API int fg_sddmm_coo_general_plan_f32(const fg_sddmm_plan *plan, const float *src, const float *dst, float *out,
+                                         int32_t F, int32_t edge_op, void *stream);
+
+/*
  * Edge softmax (no counterpart in the reference; the step between the scores of
  * multi-head SDDMM and the weights of multi-head SpMM in a GAT-style layer).
  * The edge list is the CSR one: row r's edges are [indptr[r], indptr[r+1]).

@@ -148,6 +148,47 @@ def test_elementwise_edge_function_on_a_large_edge_list():
                                rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
+def test_elementwise_edge_functions_over_row_runs(op):
+    """A row-sorted list with column blocks takes the row-run schedule (Dst tile in registers, one store per gathered
+    Src tile); one rounded operation per element, so the bits are those of the edge-parallel kernel and of numpy.
+    Feature lengths: tiles of 16, 32 and 64 floats, a partial last tile, several tiles; 30 is not a multiple of 4
+    and a shuffled list has no row runs of its own: both keep the edge-parallel kernel."""
+    from featgraph_amd import _lib
+    csr = datasets.config_graph("c2-mini").tocsr()
+    csr = scipy.sparse.vstack([csr[:50], scipy.sparse.csr_matrix((2, csr.shape[1]), dtype=csr.dtype), csr[50:]]).tocsr()
+    coo = csr.tocoo()
+    rng = np.random.default_rng(6)
+    try:
+        _lib.config_set("sddmm.blocked", 1)
+        for block_cols in (700, 64):
+            _lib.config_set("sddmm.block_cols", block_cols)
+            for F in (8, 16, 32, 64, 72, 200, 30):
+                src = rng.standard_normal((coo.shape[1], F), dtype=np.float32)
+                dst = rng.standard_normal((coo.shape[0], F), dtype=np.float32) + np.float32(3.0)
+                module = GeneralizedSDDMMhip(coo, op)
+                ph = [placeholder(src.shape), placeholder(dst.shape)]
+                assert ("row runs" in module.lower_to_ir(ph, {}, {})) == (F % 4 == 0)
+                module.build(ph, {}, {})
+                module.out_tvm.tensor.fill_(7.0)                 # every element must be written
+                out = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
+                a, b = src[coo.col], dst[coo.row]
+                assert np.array_equal(out, {"add": a + b, "sub": a - b, "mul": a * b, "div": a / b}[op]), (block_cols, F)
+        perm = rng.permutation(coo.nnz)
+        shuffled = scipy.sparse.coo_matrix((coo.data[perm], (coo.row[perm], coo.col[perm])), shape=coo.shape)
+        src = rng.standard_normal((coo.shape[1], 64), dtype=np.float32)
+        dst = rng.standard_normal((coo.shape[0], 64), dtype=np.float32) + np.float32(3.0)
+        module = GeneralizedSDDMMhip(shuffled, op)
+        ph = [placeholder(src.shape), placeholder(dst.shape)]
+        assert "row runs" not in module.lower_to_ir(ph, {}, {})
+        module.build(ph, {}, {})
+        out = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
+        assert np.array_equal(out, ref.sddmm_general(shuffled.row, shuffled.col, src, dst, op))
+    finally:
+        _lib.config_set("sddmm.blocked", -1)
+        _lib.config_set("sddmm.block_cols", 0)
+
+
 def test_bad_operator_names_and_codes():
     from featgraph_amd import _lib
     adj = reference_test_matrix("csr", seed=0)
