@@ -243,8 +243,9 @@ def main():
         a = torch.empty(n, dtype=torch.float32, device=dev).normal_()
         b = torch.empty_like(a)
         ms = timed(lambda: b.copy_(a), args.steps, args.warmup)
+        fill_ms = timed(lambda: b.fill_(1.0), args.steps, args.warmup)  # stores alone
         print(json.dumps({"kernel": "copy", "bytes_read": 4 * n, "bytes_written": 4 * n, "ms": ms,
-                          "GBps": 8 * n / ms / 1e6}))
+                          "GBps": 8 * n / ms / 1e6, "fill_ms": fill_ms, "fill_GBps": 4 * n / fill_ms / 1e6}))
         return
 
     t = time.time()
