@@ -224,3 +224,41 @@ def test_spmm_backward_is_transpose_spmm_and_sddmm(name, F):
     lhs = float((adj.astype(np.float64).dot(x.astype(np.float64)) * dout).sum())
     assert abs(lhs - float((x.astype(np.float64) * dx).sum())) <= 1e-6 * abs(lhs) + 1e-2
     assert abs(lhs - float((adj.data.astype(np.float64) * da).sum())) <= 1e-6 * abs(lhs) + 1e-2
+
+
+def _random_csr(rng, n_rows, n_cols, mean_deg, hubs):
+    deg = np.minimum(rng.poisson(mean_deg, n_rows), n_cols)
+    deg[rng.integers(0, n_rows, hubs)] = np.minimum(rng.integers(n_cols // 2, n_cols + 1, hubs), n_cols)
+    deg[rng.random(n_rows) < 0.15] = 0
+    indptr = np.zeros(n_rows + 1, dtype=np.int32)
+    np.cumsum(deg, out=indptr[1:])
+    indices = np.concatenate([np.sort(rng.choice(n_cols, d, replace=False)) for d in deg] + [np.empty(0, np.int64)])
+    vals = (rng.standard_normal(int(indptr[-1])) + 3.0).astype(np.float32)     # divisors away from zero
+    return scipy.sparse.csr_matrix((vals, indices.astype(np.int32), indptr), shape=(n_rows, n_cols))
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_structures_messages_and_reducers_under_random_schedules(seed):
+    """Seeded random matrices (empty rows, rows that fill half the columns and more), a random message and reducer,
+    random pass widths, long-run thresholds, grid sizes and kernel choice; infinities and a not-a-number among the
+    features.  Bit-exact against the checker."""
+    from featgraph_amd import _lib
+    rng = np.random.default_rng(3000 + seed)
+    n_rows, n_cols = int(rng.integers(1, 400)), int(rng.integers(1, 3000))
+    adj = _random_csr(rng, n_rows, n_cols, float(rng.choice([0.5, 3, 20, 90])), int(rng.integers(0, 4)))
+    keys = {"spmm.blocked": int(rng.integers(0, 2)), "spmm.block_cols": int(rng.choice([1, 5, 64, 300, 1 << 20])),
+            "spmm.multi_long": int(rng.choice([0, 4, 64, 700])), "spmm.multi_blocks": int(rng.choice([0, 1, 2])),
+            "spmm.relay": int(seed % 3 != 0), "spmm.general_multi": int(seed % 4 != 0)}
+    try:
+        for k, v in keys.items():
+            _lib.config_set(k, v)
+        for F in rng.choice([1, 4, 8, 20, 24, 32, 36, 64, 100, 128, 200], 4, replace=False):
+            msg, reduce = str(rng.choice(MSGS)), str(rng.choice(REDUCES))
+            feat = rng.standard_normal((n_cols, int(F))).astype(np.float32)
+            feat[rng.integers(0, n_cols, 3), rng.integers(0, int(F), 3)] = [np.inf, -np.inf, np.nan]
+            out = _run_general_spmm(adj, feat, msg, reduce)
+            want = ref.spmm_general(adj.indptr, adj.indices, adj.data, feat, msg, reduce)
+            assert np.array_equal(out, want, equal_nan=True), (seed, int(F), msg, reduce, keys)
+    finally:
+        for k in keys:
+            _lib.config_set(k, 0 if k in ("spmm.block_cols", "spmm.multi_long", "spmm.multi_blocks") else -1)
