@@ -7,8 +7,8 @@ import numpy as np
 import pytest
 
 from featgraph_amd import datasets, nd, placeholder
-from featgraph_amd.module import (MultiHeadSDDMMhip, MultiHeadSDDMMSoftmaxhip, MultiHeadSpMMhip, VanillaSDDMMhip,
-                                  VanillaSpMMhip)
+from featgraph_amd.module import (GeneralizedSDDMMhip, GeneralizedSpMMhip, MultiHeadSDDMMhip, MultiHeadSDDMMSoftmaxhip,
+                                  MultiHeadSpMMhip, VanillaSDDMMhip, VanillaSpMMhip)
 from oracle import ref
 
 pytestmark = pytest.mark.gpu
@@ -195,6 +195,42 @@ def test_c3_sddmm_on_a_shuffled_edge_list(c2, F):
     sorted_module.build(ph, {}, {})
     base = sorted_module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
     assert np.array_equal(out, base[perm])
+
+
+@pytest.mark.parametrize("msg,reduce,F", [("sub", "mean", 32), ("div", "max", 128), ("copy_u", "min", 64)])
+def test_c2_generalised_spmm_bit_exact(c2, msg, reduce, F):
+    """The several-rows-per-wave kernel with a message and a reducer in place of the multiply-add, at full size:
+    tiles of 32 and 64 floats, several tiles, long runs, the division of the mean."""
+    adj = c2
+    n = adj.shape[0]
+    vals = adj.data + np.float32(0.5)                                   # divisors away from zero
+    module = GeneralizedSpMMhip(type(adj)((vals, adj.indices, adj.indptr), shape=adj.shape), msg, reduce)
+    ph = [placeholder((n, F))]
+    text = module.lower_to_ir(ph, {}, {})
+    _say("generalised SpMM c2 %s/%s F=%d: %s" % (msg, reduce, F, text))
+    assert "rows-per-wave" in text
+    module.build(ph, {}, {})
+    feat = datasets.spmm_operands(adj, F)
+    out = module.run([nd.array(feat, module.ctx)]).asnumpy()
+    assert np.array_equal(out, ref.spmm_general(adj.indptr, adj.indices, vals, feat, msg, reduce))
+
+
+def test_c3_elementwise_edge_function_over_row_runs(c2):
+    """Out[e, :] = Src[col[e], :] * Dst[row[e], :] on the full edge list (a 14.7 GB result at 32 floats), checked on
+    the first and last two million edges against numpy."""
+    coo = c2.tocoo()
+    n, F = coo.shape[0], 32
+    module = GeneralizedSDDMMhip(coo, "mul")
+    ph = [placeholder((n, F)), placeholder((n, F))]
+    text = module.lower_to_ir(ph, {}, {})
+    _say("elementwise SDDMM c3 mul F=%d: %s" % (F, text))
+    assert "row runs" in text
+    module.build(ph, {}, {})
+    src, dst = datasets.sddmm_operands(coo, F)
+    out = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).tensor
+    m = 2_000_000
+    for sl in (slice(0, m), slice(coo.nnz - m, coo.nnz)):
+        assert np.array_equal(out[sl].cpu().numpy(), src[coo.col[sl]] * dst[coo.row[sl]])
 
 
 @pytest.mark.parametrize("D", [32, 64])
