@@ -635,9 +635,9 @@ int fg_spmm_csr_general_f32(const fg_spmm_plan *plan, const float *feat, const f
     return fg::fail(FG_EINVAL, "feat or edge values are null");
   if (plan->n_rows == 0) return FG_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  // The several-rows-per-wave kernel takes the call where it would take the plain operator (tiles of 32 and 64
-  // floats): same records, same passes, the message and the reducer in place of the multiply-add; the mean is
-  // the sum followed by one division per element.
+  // The several-rows-per-wave kernel takes the call where it would take the plain operator: same records, same
+  // passes, the message and the reducer in place of the multiply-add; the mean is the sum followed by one
+  // division per element.
   if (plan->nnz > 0 && fg::config().spmm_general_multi != 0) {
     fg::SpmmArgs a;
     fg::SpmmShape s;

@@ -1,5 +1,5 @@
 // The several-rows-per-wave SpMM kernel as the generalised operator with the message FG_MSG_SUB (three reducers, tiles
-// of 32 and 64 floats).
+// of 16, 32 and 64 floats).
 #include "spmm_multi_kernel.hpp"
 
 namespace fg {

@@ -462,20 +462,20 @@ int launch_multi(const SpmmArgs &a, int64_t blocks, bool buf, bool u24, hipStrea
   return FG_OK;
 }
 
-// The generalised operator with message MSG: tiles of 32 or 64 floats, reducer a.reduce (sum / max / min).
+// The generalised operator with message MSG and reducer RED, tile width by feature length as for the plain one.
+template <int RED, int MSG>
+int launch_multi_general_tile(const SpmmArgs &a, int64_t blocks, hipStream_t stream) {
+  if (a.F <= 16) return launch_multi<4, RED, MSG>(a, blocks, true, true, stream);
+  if (a.F <= 32) return launch_multi<8, RED, MSG>(a, blocks, true, true, stream);
+  return launch_multi<16, RED, MSG>(a, blocks, true, true, stream);
+}
+
 template <int MSG>
 int launch_multi_general(const SpmmArgs &a, int64_t blocks, hipStream_t stream) {
-  const bool narrow = a.F <= 32;
   switch (a.reduce) {
-    case FG_REDUCE_SUM:
-      return narrow ? launch_multi<8, FG_REDUCE_SUM, MSG>(a, blocks, true, true, stream)
-                    : launch_multi<16, FG_REDUCE_SUM, MSG>(a, blocks, true, true, stream);
-    case FG_REDUCE_MAX:
-      return narrow ? launch_multi<8, FG_REDUCE_MAX, MSG>(a, blocks, true, true, stream)
-                    : launch_multi<16, FG_REDUCE_MAX, MSG>(a, blocks, true, true, stream);
-    case FG_REDUCE_MIN:
-      return narrow ? launch_multi<8, FG_REDUCE_MIN, MSG>(a, blocks, true, true, stream)
-                    : launch_multi<16, FG_REDUCE_MIN, MSG>(a, blocks, true, true, stream);
+    case FG_REDUCE_SUM: return launch_multi_general_tile<FG_REDUCE_SUM, MSG>(a, blocks, stream);
+    case FG_REDUCE_MAX: return launch_multi_general_tile<FG_REDUCE_MAX, MSG>(a, blocks, stream);
+    case FG_REDUCE_MIN: return launch_multi_general_tile<FG_REDUCE_MIN, MSG>(a, blocks, stream);
   }
   return fail(FG_EINVAL, "reduce = %d has no several-rows-per-wave kernel", a.reduce);
 }

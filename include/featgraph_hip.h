@@ -132,7 +132,7 @@ FG_API int fg_spmm_csr_noalloc_f32(int64_t n_rows, int64_t n_cols, int64_t nnz, 
  * message and per fold step, so (MUL, SUM) equals fg_spmm_csr_f32 bit for bit.
  * vals may be null for FG_MSG_COPY_U.  Runs the kernel of fg_spmm_csr_f32 with
  * the message and the reducer in place of the multiply-add where that kernel
- * applies (feature lengths that are multiples of 4 above 16), a row-slot kernel
+ * applies (feature lengths that are multiples of 4), a row-slot kernel
  * otherwise; one launch per column block of the plan (one launch over whole
  * rows when the plan has no blocks), MEAN one more for the division.  The
  * partial fold of a row is carried in `out` between launches, so `out` must
