@@ -92,6 +92,7 @@ def test_error_codes_of_the_later_entry_points_without_a_device():
     assert L.fg_sddmm_coo_general_f32(4, 8, 8, 8, 8, 8, 4, 7, None) == -1                # no such edge function
     assert L.fg_sddmm_coo_general_f32(-1, 8, 8, 8, 8, 8, 4, 1, None) == -1
     assert L.fg_sddmm_coo_general_f32(0, None, None, None, None, None, 4, 2, None) == 0  # empty edge list
+    assert L.fg_sddmm_coo_general_plan_f32(None, 8, 8, 8, 4, 1, None) == -1              # no plan
     # edge softmax
     assert L.fg_edge_softmax_csr_f32(-1, None, None, None, 8, None) == -1
     assert L.fg_edge_softmax_csr_f32(4, None, None, None, 8, None) == -1                 # null data
