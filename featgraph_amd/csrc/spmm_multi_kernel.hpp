@@ -12,9 +12,11 @@
 // for bit, as in the other kernels and in the reference's loop nest
 // (op/vanilla_spmm.py:46-56).
 //
-// Work comes as records {first nonzero, one past the last, row}, one per row
-// and column-block pass, which the plan sorts by descending run length inside
-// each pass: the rows that share a wave then finish together (the wave runs
+// Work comes as records {first nonzero, one past the last, row, first nonzero
+// in the CSR arrays}, one per row and column-block pass, which the plan sorts by
+// descending run length inside each pass; the first two index either the CSR
+// column ids or the plan's copy of them in the records' own order, and the
+// values always sit at the CSR position.  The rows that share a wave then finish together (the wave runs
 // until its longest row is done; shorter ones skip the adds, and their idle
 // gathers re-read row 0 of the band and are dropped).  A lane holds the ids and
 // values of four consecutive nonzeros, so one 16-byte load per lane brings 4*G
@@ -24,6 +26,10 @@
 // of ids is asked for behind the current batch's first gathers (loads return in
 // order, so the adds wait only for the gathers).  Runs of kLongRun nonzeros or
 // more take the one-wave-per-run path below instead.
+//
+// RED / MSG turn the multiply-add into the generalised operator (README.md:6 of the reference): term =
+// MSG(feature, value), folded with RED in the same order; a picking reducer (max / min) takes a row's first
+// term as it is, which a run recognises by its CSR position being indptr[row].
 //
 // This file holds the kernel and its launcher as templates; spmm_multi.hip instantiates the plain operator and
 // spmm_multi_general_*.hip the generalised one, one message per file (each instance is a large kernel, and the
@@ -37,7 +43,6 @@
 
 namespace fg {
 namespace {
-
 
 // Runs of at least this many nonzeros go to the one-wave-per-run path (spmm.multi_long overrides).
 constexpr uint32_t kLongRun = 512;
