@@ -8,7 +8,11 @@ of the Reddit graph that the reference's benchmark scripts load,
 benchmark/bench_vanilla_spmm.py:77-79), float32, synthetic and seeded.  One
 "step" is one vanilla CSR SpMM at feature length 64 with every operand already
 resident in device memory.  W warm-up steps, then exactly K steps are timed
-between two events on the launch stream; the printed JSON line carries
+between two events on the launch stream.  The LAST line of stdout is one short
+JSON object (under 1.5 KB: metric, value, roofline, cpu_baseline, parity); every
+other row (feature-length sweep, multi-head operators, probes, per-setting CPU
+timings) is printed earlier, one compact JSON object per line on stderr, and
+the whole record is also written to gpurun_out/bench_detail.json.  The record carries
 
   value        SpMM GFLOP/s (2*nnz*F flops per step)
   roofline     `achieved` / `frac`: algorithmic gather-model bytes (nnz*(8+4F) + rows*(4+4F)) over the measured
@@ -119,6 +123,77 @@ def cpu_model():
     except OSError:
         pass
     return "unknown"
+
+
+def _sig(x, digits=5):
+    """Floats shortened to `digits` significant digits (the short line only; the detail record keeps full precision)."""
+    if isinstance(x, float):
+        return float("%.*g" % (digits, x))
+    if isinstance(x, dict):
+        return {k: _sig(v, digits) for k, v in x.items()}
+    if isinstance(x, (list, tuple)):
+        return [_sig(v, digits) for v in x]
+    return x
+
+
+HEADLINE_LIMIT = 1500
+
+
+def headline(result, detail_path=None):
+    """The short record that ends stdout: what a harness reads, nothing else.  Built from the detail record."""
+    r = result["roofline"]
+    roof = {k: r.get(k) for k in ("bound", "achieved", "peak", "unit", "frac", "frac_bounded", "traffic",
+                                  "traffic_source", "algorithmic_bytes", "kernel", "dispatches_per_launch",
+                                  "hbm_frac_compulsory", "frac_of_gather_ceiling")}
+    line = {k: result.get(k) for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
+                                       "higher_is_better", "scaling", "vs_baseline", "dtype", "data", "config")}
+    line["roofline"] = roof
+    if result.get("roofline_hbm_bound_config"):
+        line["roofline_hbm_bound_config"] = result["roofline_hbm_bound_config"]
+    c = result.get("cpu_baseline")
+    if c:
+        line["cpu_baseline"] = {k: c.get(k) for k in ("value", "unit", "cores", "kind", "seconds", "cpu_model",
+                                                      "best_num_feat_partitions", "sample")}
+    p = result.get("parity")
+    if p is not None:
+        line["parity"] = all(v for v in p.values() if isinstance(v, bool))
+    if detail_path:
+        line["detail"] = detail_path
+    return _sig(line)
+
+
+def headline_line(result, detail_path=None):
+    line = json.dumps(headline(result, detail_path), separators=(",", ":"))
+    if len(line) >= HEADLINE_LIMIT:
+        raise RuntimeError("the headline line grew to %d characters (limit %d)" % (len(line), HEADLINE_LIMIT))
+    return line
+
+
+def emit(result):
+    """Detail rows to stderr (one compact JSON object per line), the whole record to a file, the headline last on stdout."""
+    def row(tag, obj):
+        print(json.dumps({"detail": tag, **_sig(obj, 6)}, separators=(",", ":")), file=sys.stderr)
+
+    for r in result.get("sweep", []):
+        row("sweep", r)
+    for r in result.get("multi_head", {}).get("rows", []):
+        row("multi_head", r)
+    for key in ("pcie_inclusive", "small_graph", "cpu_baseline", "cpu_baseline_sddmm", "parity", "plan_seconds"):
+        if key in result:
+            row(key, result[key] if isinstance(result[key], dict) else {"value": result[key]})
+    row("roofline", result["roofline"])
+    row("launch", {"text": result.get("launch")})
+    detail_path = None
+    try:
+        out_dir = os.path.join(ROOT, "gpurun_out")
+        os.makedirs(out_dir, exist_ok=True)
+        with open(os.path.join(out_dir, "bench_detail.json"), "w") as f:
+            json.dump(result, f, indent=1)
+        detail_path = "gpurun_out/bench_detail.json"
+    except OSError:
+        pass
+    sys.stderr.flush()
+    print(headline_line(result, detail_path), flush=True)
 
 
 def log(*a):
@@ -440,12 +515,17 @@ def main():
     traffic, traffic_source = committed_traffic("spmm", args.graph, F)
     probe = gather_probe(feat.tensor, nnz) if args.only == "all" else None
     probe_hit = gather_probe_at_hit_rate(feat.tensor, nnz, "spmm", F) if args.only == "all" else None
+    launch_text = spmm.lower_to_ir([placeholder((n_cols, F))], {}, {})
+    m_pass = re.search(r"(\d+) launch", launch_text)
+    launch_dispatches = int(m_pass.group(1)) if m_pass else None
     roofline = {
         "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
         "traffic": traffic, "traffic_source": traffic_source,
         "algorithmic_bytes": alg, "kernel": "spmm (CSR, feat-len %d)" % F, "launch_ms": ms,
         "compulsory_bytes": b_min, "hbm_frac_compulsory": b_min / ms / 1e6 / HBM_PEAK_GBPS,
         "l2_fabric_frac": (traffic / ms / 1e6 / HBM_PEAK_GBPS) if traffic else None,
+        "frac_bounded": (traffic / ms / 1e6 / HBM_PEAK_GBPS) if traffic else None,
+        "dispatches_per_launch": launch_dispatches,
         "gather_ceiling": probe, "frac_of_gather_ceiling": (probe["ms"] / ms) if probe else None,
         "gather_at_the_operators_l2_hit_rate": probe_hit,
         "frac_of_gather_at_the_operators_l2_hit_rate": (probe_hit["ms"] / ms) if probe_hit else None,
@@ -458,18 +538,18 @@ def main():
                 "operator launch. `traffic` is read from the committed profile named in traffic_source, not "
                 "measured in this run."}
     result = {
-        "metric": "SpMM GFLOP/s (vanilla CSR, fp32, feat-len %d) with achieved algorithmic GB/s vs HBM roofline" % F,
+        "metric": "SpMM GFLOP/s (vanilla CSR, fp32, feat-len %d)" % F,
         "value": flops / ms / 1e6, "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
-        "data": "synthetic (seeded power-law graph, N(0,1) features)",
+        "data": "synthetic",
         "config": {"workload": "%s: vanilla CSR SpMM, %d vertices, %d nonzeros, feat-len %d" % (
             args.graph, n_rows, nnz, F), "graph_checksum": datasets.structure_checksum(adj)},
         "roofline": roofline,
-        "launch": spmm.lower_to_ir([placeholder((n_cols, F))], {}, {}),
+        "launch": launch_text,
         "plan_seconds": plan_seconds,
     }
     if args.only == "spmm":
-        print(json.dumps(result))
+        print(headline_line(result))
         return
 
     # ---- the same step for a caller that starts from host memory (never `value`): pinned upload of the
@@ -648,6 +728,12 @@ def main():
             torch.cuda.empty_cache()
             log("%s D=64: %.3f ms (scores + softmax, then multi-head SpMM: %.3f ms)" % (
                 kind, mh[-1]["ms"], mh[-1]["chain_ms"]))
+        hb = next(r for r in mh if r["op"] == "mh_spmm")
+        result["roofline_hbm_bound_config"] = {
+            "workload": "c5: multi-head CSR SpMM, %d vertices, %d edges, H=8, D=64" % (big.shape[0], big.nnz),
+            "ms": hb["ms"], "algorithmic_bytes": hb["algorithmic_bytes"], "achieved": hb["alg_GBps"],
+            "frac": hb["frac"], "traffic": hb.get("traffic"), "frac_traffic": hb.get("hbm_frac_traffic"),
+            "parity": (hb.get("parity") or {}).get("bit_exact_vs_cpu_checker")}
         result["multi_head"] = {"graph": "c4: %d vertices, %d edges" % (big.shape[0], big.nnz), "rows": mh,
                                 "note": "1.25 - 5 GB of features and mean degree 25: nearly every neighbour gather "
                                         "goes to HBM.  `frac` is algorithmic bytes / time / 8 TB/s (above 1 for SDDMM "
@@ -717,10 +803,8 @@ def main():
             "cpu_model": cpu_model(), "best_num_feat_partitions": best,
             "value_at_num_feat_partitions_1": flops / per_p[1]["seconds"] / 1e9,
             "per_num_feat_partitions": {str(p): v for p, v in per_p.items()},
-            "sample": "the whole workload (%s, feat-len %d): restated TVM x86 nest with both layout transforms, "
-                      "num_feat_partitions swept over %s as benchmark/bench_vanilla_spmm.py:37 does (best: %d), "
-                      "OpenMP static rows on %d threads, mean of %d run(s) after one warm-up per setting" % (
-                          args.graph, F, sorted(per_p), best, cores, per_p[best]["runs"])}
+            "sample": "whole workload, restated x86 nest, num_feat_partitions in %s, mean of %d run(s)" % (
+                sorted(per_p), per_p[best]["runs"])}
         result["parity"] = {"spmm_bit_exact_vs_cpu_restatement": bool(np.array_equal(gpu_out, cpu_out)),
                             "spmm_max_abs_diff": float(np.max(np.abs(gpu_out - cpu_out)))}
         # distance of the float32 result (the reference's summation order) from the exact sum, by row degree
@@ -775,7 +859,7 @@ def main():
         result["tvm_available"] = True
     except Exception:
         result["tvm_available"] = False
-    print(json.dumps(result))
+    emit(result)
 
 
 if __name__ == "__main__":
