@@ -20,7 +20,7 @@
 // had to refuse for lack of a cross-block reduction; launches on one stream are
 // ordered, so the running sums need no atomics).  Every Out[e] is written by one
 // lane per tile, at the edge's original position: results are deterministic.
-#include <hipcub/hipcub.hpp>
+#include <rocprim/device/device_radix_sort.hpp>
 
 #include "common.hpp"
 
@@ -103,12 +103,12 @@ int sddmm_blocks_build(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_
     err = hipGetLastError();
   }
   if (err == hipSuccess)
-    err = hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, keys, keys_sorted, ids, out->pos_p,
-                                             static_cast<int>(nnz), 0, bits, nullptr);
+    err = rocprim::radix_sort_pairs(nullptr, tmp_bytes, keys, keys_sorted, ids, out->pos_p,
+                                             static_cast<unsigned>(nnz), 0, bits, nullptr);
   if (err == hipSuccess) err = hipMalloc(&tmp, tmp_bytes ? tmp_bytes : 1);
   if (err == hipSuccess)  // LSD radix sort: stable, so edges with equal keys keep the caller's order
-    err = hipcub::DeviceRadixSort::SortPairs(tmp, tmp_bytes, keys, keys_sorted, ids, out->pos_p,
-                                             static_cast<int>(nnz), 0, bits, nullptr);
+    err = rocprim::radix_sort_pairs(tmp, tmp_bytes, keys, keys_sorted, ids, out->pos_p,
+                                             static_cast<unsigned>(nnz), 0, bits, nullptr);
   if (err == hipSuccess) {
     const int grid = static_cast<int>(std::min<int64_t>((nnz + 255) / 256, 65536));
     gather_edges_kernel<<<dim3(grid), dim3(256)>>>(row, col, out->pos_p, nnz, out->row_p, out->col_p);

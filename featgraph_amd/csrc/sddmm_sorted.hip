@@ -5,7 +5,7 @@
 // row-run kernel over the copy -- the dot products land in sorted order in memory the plan owns -- and brings
 // them back to the caller's positions: a fixed permutation of nnz floats, done as two permutations that each stay
 // inside blocks of 32768 elements (below), or as one gather when that routing could not be built.
-#include <hipcub/hipcub.hpp>
+#include <rocprim/device/device_radix_sort.hpp>
 
 #include "common.hpp"
 
@@ -151,10 +151,10 @@ hipError_t regroup_build(const int32_t *pos, int64_t nnz, SddmmSorted *out) {
   if (err == hipSuccess) err = hipMalloc(&out->b_local, n * sizeof(uint16_t));
   if (err == hipSuccess) err = hipMalloc(&out->from, n * sizeof(int32_t));
   if (err == hipSuccess)
-    err = hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_a, keys, keys_sorted, ids, order_a, static_cast<int>(nnz), 0,
+    err = rocprim::radix_sort_pairs(nullptr, tmp_a, keys, keys_sorted, ids, order_a, static_cast<unsigned>(nnz), 0,
                                              2 * block_bits, nullptr);
   if (err == hipSuccess)
-    err = hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_b, keys, keys_sorted, ids, out->from, static_cast<int>(nnz), 0,
+    err = rocprim::radix_sort_pairs(nullptr, tmp_b, keys, keys_sorted, ids, out->from, static_cast<unsigned>(nnz), 0,
                                              block_bits, nullptr);
   if (err == hipSuccess) err = hipMalloc(&tmp, std::max<size_t>(std::max(tmp_a, tmp_b), 1));
   if (err == hipSuccess) {
@@ -162,14 +162,14 @@ hipError_t regroup_build(const int32_t *pos, int64_t nnz, SddmmSorted *out) {
     err = hipGetLastError();
   }
   if (err == hipSuccess)  // source block above destination block; stable, so a piece keeps the sorted order
-    err = hipcub::DeviceRadixSort::SortPairs(tmp, tmp_a, keys, keys_sorted, ids, order_a, static_cast<int>(nnz), 0,
+    err = rocprim::radix_sort_pairs(tmp, tmp_a, keys, keys_sorted, ids, order_a, static_cast<unsigned>(nnz), 0,
                                              2 * block_bits, nullptr);
   if (err == hipSuccess) {
     regroup_a_kernel<<<dim3(grid), dim3(256)>>>(order_a, pos, nnz, out->a_local, keys, ids, b_local_of_place);
     err = hipGetLastError();
   }
   if (err == hipSuccess)  // by destination block; stable, so a block's pieces come by ascending place
-    err = hipcub::DeviceRadixSort::SortPairs(tmp, tmp_b, keys, keys_sorted, ids, out->from, static_cast<int>(nnz), 0,
+    err = rocprim::radix_sort_pairs(tmp, tmp_b, keys, keys_sorted, ids, out->from, static_cast<unsigned>(nnz), 0,
                                              block_bits, nullptr);
   if (err == hipSuccess) {
     regroup_b_kernel<<<dim3(grid), dim3(256)>>>(out->from, b_local_of_place, nnz, out->b_local);
@@ -246,11 +246,11 @@ int sddmm_sorted_build(int64_t nnz, int64_t n_rows, int64_t n_cols, const int32_
   }
   if (err == hipSuccess) err = hipMemcpy(&bad, flag, sizeof(int), hipMemcpyDeviceToHost);
   if (err == hipSuccess && !bad)
-    err = hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, keys, keys_sorted, ids, pos, static_cast<int>(nnz), 0,
+    err = rocprim::radix_sort_pairs(nullptr, tmp_bytes, keys, keys_sorted, ids, pos, static_cast<unsigned>(nnz), 0,
                                              row_bits + col_bits, nullptr);
   if (err == hipSuccess && !bad) err = hipMalloc(&tmp, tmp_bytes ? tmp_bytes : 1);
   if (err == hipSuccess && !bad)  // stable: edges listed twice keep the caller's order
-    err = hipcub::DeviceRadixSort::SortPairs(tmp, tmp_bytes, keys, keys_sorted, ids, pos, static_cast<int>(nnz), 0,
+    err = rocprim::radix_sort_pairs(tmp, tmp_bytes, keys, keys_sorted, ids, pos, static_cast<unsigned>(nnz), 0,
                                              row_bits + col_bits, nullptr);
   if (err == hipSuccess && !bad) {
     sorted_edges_kernel<<<dim3(grid), dim3(256)>>>(keys_sorted, pos, nnz, col_bits, out->row_s, out->col_s, out->where);

@@ -1,7 +1,8 @@
 // CSR SpMM, several rows per wave with 16-byte gathers (gfx950): the plan's run records, the re-laid column
 // ids, and the launch of the kernel of spmm_multi_kernel.hpp for the plain operator; the generalised operator's
 // instances live in spmm_multi_general_*.hip.
-#include <hipcub/hipcub.hpp>
+#include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/device/device_scan.hpp>
 
 #include "spmm_multi_kernel.hpp"
 
@@ -70,7 +71,7 @@ hipError_t relay_build(const int32_t *indices, int64_t nnz, int64_t n_rec, Multi
   hipError_t err = hipMalloc(&len, n_rec * sizeof(int32_t));
   if (err == hipSuccess) err = hipMalloc(&first_p, n_rec * sizeof(int32_t));
   if (err == hipSuccess)
-    err = hipcub::DeviceScan::ExclusiveSum(nullptr, tmp_bytes, len, first_p, static_cast<int>(n_rec), nullptr);
+    err = rocprim::exclusive_scan(nullptr, tmp_bytes, len, first_p, int32_t(0), static_cast<size_t>(n_rec), rocprim::plus<int32_t>(), nullptr);
   if (err == hipSuccess) err = hipMalloc(&tmp, tmp_bytes ? tmp_bytes : 1);
   const unsigned grid = static_cast<unsigned>((n_rec + 255) / 256);
   if (err == hipSuccess) {
@@ -78,7 +79,7 @@ hipError_t relay_build(const int32_t *indices, int64_t nnz, int64_t n_rec, Multi
     err = hipGetLastError();
   }
   if (err == hipSuccess)
-    err = hipcub::DeviceScan::ExclusiveSum(tmp, tmp_bytes, len, first_p, static_cast<int>(n_rec), nullptr);
+    err = rocprim::exclusive_scan(tmp, tmp_bytes, len, first_p, int32_t(0), static_cast<size_t>(n_rec), rocprim::plus<int32_t>(), nullptr);
   if (err == hipSuccess) err = hipMemcpy(&last[0], first_p + n_rec - 1, sizeof(int32_t), hipMemcpyDeviceToHost);
   if (err == hipSuccess) err = hipMemcpy(&last[1], len + n_rec - 1, sizeof(int32_t), hipMemcpyDeviceToHost);
   const int64_t total = static_cast<int64_t>(last[0]) + last[1];
@@ -139,8 +140,8 @@ int multi_runs_build(const int32_t *seg, const int32_t *row_order, const int32_t
   if (err == hipSuccess) err = hipMalloc(&ids, n * sizeof(int32_t));
   if (err == hipSuccess) err = hipMalloc(&ids_sorted, n * sizeof(int32_t));
   if (err == hipSuccess)
-    err = hipcub::DeviceRadixSort::SortPairsDescending(nullptr, tmp_bytes, keys, keys_sorted, ids, ids_sorted,
-                                                       static_cast<int>(n_rows), 0, 32, nullptr);
+    err = rocprim::radix_sort_pairs_desc(nullptr, tmp_bytes, keys, keys_sorted, ids, ids_sorted,
+                                                       static_cast<unsigned>(n_rows), 0, 32, nullptr);
   if (err == hipSuccess) err = hipMalloc(&tmp, tmp_bytes ? tmp_bytes : 1);
   const unsigned grid = static_cast<unsigned>((n_rows + 255) / 256);
   for (int p = 0; p < passes && err == hipSuccess; ++p) {
@@ -150,8 +151,8 @@ int multi_runs_build(const int32_t *seg, const int32_t *row_order, const int32_t
     count_long_runs_kernel<<<dim3(grid), dim3(256)>>>(keys, n_rows, long_run, counts + p);
     err = hipGetLastError();
     if (err == hipSuccess)  // LSD radix sort: stable
-      err = hipcub::DeviceRadixSort::SortPairsDescending(tmp, tmp_bytes, keys, keys_sorted, ids, ids_sorted,
-                                                         static_cast<int>(n_rows), 0, 32, nullptr);
+      err = rocprim::radix_sort_pairs_desc(tmp, tmp_bytes, keys, keys_sorted, ids, ids_sorted,
+                                                         static_cast<unsigned>(n_rows), 0, 32, nullptr);
     if (err == hipSuccess) {
       run_records_kernel<<<dim3(grid), dim3(256)>>>(lo, hi, row_order, ids_sorted, n_rows, out->rec + p * n);
       err = hipGetLastError();
