@@ -41,7 +41,7 @@ NoallocScratch *g_scratch[kMaxDevices] = {};  // device address of `scratch` on 
 
 // The array's name is only a handle on the host; kernels and fills need its device address, which differs
 // from GPU to GPU.  Called with the target device current.
-int scratch_address(NoallocScratch **out) {
+int scratch_address(NoallocScratch **out, hipStream_t stream) {
   int device = -1;
   FG_HIP_TRY(hipGetDevice(&device));
   if (device < 0 || device >= kMaxDevices)
@@ -49,6 +49,13 @@ int scratch_address(NoallocScratch **out) {
                     kMaxDevices);
   std::lock_guard<std::mutex> lock(g_mutex);
   if (!g_scratch[device]) {
+    // the lookup may load the library's code object on this GPU: not something to do while `stream` records a graph
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) (void)hipGetLastError();
+    if (capturing != hipStreamCaptureStatusNone)
+      return fg::fail(FG_EUNSUPPORTED,
+                      "the first fg_spmm_csr_noalloc_f32 call on a GPU must not be under stream capture: call it "
+                      "once eagerly on device %d before recording it", device);
     void *ptr = nullptr;
     FG_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
     if (!ptr) return fg::fail(FG_EHIP, "hipGetSymbolAddress returned a null address for the schedule array");
@@ -126,8 +133,8 @@ extern "C" int fg_spmm_csr_noalloc_f32(int64_t n_rows, int64_t n_cols, int64_t n
   if (n_rows == 0) return FG_OK;
 
   NoallocScratch *s = nullptr;
-  if (int rc = scratch_address(&s)) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (int rc = scratch_address(&s, st)) return rc;
   const int32_t n = static_cast<int32_t>(n_rows);
   const unsigned grid = static_cast<unsigned>(std::min<int64_t>((n_rows + 255) / 256, 2048));
   clear_counters_kernel<<<dim3(1), dim3(kCounterInts), 0, st>>>(s->counters);

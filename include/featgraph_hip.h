@@ -112,6 +112,10 @@ FG_API int fg_spmm_csr_f32(const fg_spmm_plan *plan, const float *feat, const fl
  * hipFree, copies nothing and never synchronises.  Every call on a GPU uses
  * that GPU's one array: calls that overlap in time on the same GPU (two
  * streams, two threads) race on it and must be serialised by the caller.
+ * The array's device address is looked up at the first call on each GPU, and
+ * that lookup must not happen under stream capture: make one eager call per
+ * GPU before recording the entry point into a HIP graph.  A first call that
+ * finds `stream` capturing returns FG_EUNSUPPORTED and enqueues nothing.
  * indptr CONTENTS are the caller's contract (non-decreasing, 0 .. nnz); rows
  * whose bounds are out of range come out as zeros.
  */
@@ -304,7 +308,14 @@ FG_API int fg_sddmm_coo_mh_f32(int64_t nnz, const int32_t *row, const int32_t *c
 FG_API int fg_check_indices(int64_t n, const int32_t *idx, int64_t bound, int64_t *n_bad, void *stream);
 
 /*
- * Measurement aid (no counterpart in the reference): the gather pattern of the
+ * ---- fg_probe_*: measurement aids, NOT part of the operator API ------------
+ * The seven fg_probe_* entry points below exist for the benchmark only (bare
+ * gather / store patterns that price what the memory system does); no module
+ * class calls them, they have no counterpart in the reference, and they may
+ * change or go away without notice.  A binding for the operators leaves them
+ * out.
+ *
+ * The gather pattern of the
  * SpMM / SDDMM kernels with everything else left out.  Per feature tile of
  * `tile` floats (16, 32 or 64; F a multiple of it) it gathers about n_gathers
  * random rows of feat [n_rows, F] with 16-byte loads, tile/4 lanes per row,
