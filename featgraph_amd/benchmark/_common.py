@@ -12,13 +12,23 @@ def parser(description, matrix_format):
                      help="adjacency matrix in %s format stored as a scipy .npz file" % matrix_format)
     src.add_argument("--synthetic", type=str, help="name of a seeded synthetic graph (c1, c2, c4, c2-mini, c4-mini)")
     ap.add_argument("--feat-len", type=int, default=128, help="the feature length")
-    ap.add_argument("--target", type=str, default="hip", choices=["hip"],
-                    help="only the HIP target exists in this package")
+    ap.add_argument("--target", type=str, default="hip", choices=["hip", "cuda", "x86"],
+                    help="hip, or cuda (the reference's spelling of the GPU target, benchmark/bench_vanilla_spmm.py:"
+                         "72-75; same as hip here, as featgraph.module.VanillaSpMMcuda is VanillaSpMMhip); x86 is "
+                         "refused: this package has no CPU path")
     ap.add_argument("--num-runs", type=int, default=5, help="timed runs after one warm-up")
     return ap
 
 
+def check_target(args):
+    """The reference's --target spellings: cuda runs the HIP target; x86 has no counterpart and says so."""
+    if args.target == "x86":
+        raise SystemExit("--target x86: this package has only the GPU path (use --target hip or cuda)")
+    return "hip"
+
+
 def load_adjacency(args, matrix_format):
+    check_target(args)
     if args.dataset:
         adj = scipy.sparse.load_npz(args.dataset)
         assert adj.format == matrix_format, "expected a %s matrix, got %s" % (matrix_format, adj.format)

@@ -134,8 +134,8 @@ def c3_sddmm_module(c2):
 
 @pytest.mark.parametrize("F", [32, 128, 256, 512])
 def test_c2_spmm_bit_exact_at_every_swept_feature_length(c2, c2_spmm_module, F):
-    """Covers what only happens at full size: 15 column-block passes x F/64 tiles with carried sums, the
-    32768-column passes of the 32-float tile, more long runs than the workgroup clamp, 100 MB run tables."""
+    """Covers what only happens at full size: one launch per column-block pass over every feature tile with carried
+    sums, the wider passes of the narrower tiles, more long runs than the workgroup clamp, 100 MB run tables."""
     adj, module = c2, c2_spmm_module
     n = adj.shape[0]
     _say("SpMM c2 F=%d through VanillaSpMMhip: %s" % (F, module.lower_to_ir([placeholder((n, F))], {}, {})))

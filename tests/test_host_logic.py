@@ -141,3 +141,13 @@ def test_reference_import_paths_resolve_to_this_implementation():
     assert util_convert_csr_to_dds is featgraph_amd.util.util_convert_csr_to_dds
     assert util_partition_adj_coo_2d is featgraph_amd.util.util_partition_adj_coo_2d
     assert featgraph.placeholder is placeholder and featgraph.nd is featgraph_amd.nd
+
+
+def test_benchmark_commands_take_the_reference_target_spellings():
+    """benchmark/bench_vanilla_spmm.py:72-75 passes --target x86 | cuda: cuda is the GPU target here, x86 is refused."""
+    from featgraph_amd.benchmark import _common as B
+    ap = B.parser("x", "csr")
+    for spelling in ("hip", "cuda"):
+        assert B.check_target(ap.parse_args(["--synthetic", "c1", "--target", spelling])) == "hip"
+    with pytest.raises(SystemExit):
+        B.check_target(ap.parse_args(["--synthetic", "c1", "--target", "x86"]))
