@@ -80,6 +80,7 @@ struct fg_sddmm_plan {
   // built; the row-run kernel writes its results in that order and a gather returns them to the caller's.
   fg::SddmmSorted sorted;
   bool input_row_sorted = false;  // the caller's own list has ascending row ids (indptr then describes it too)
+  const char *no_row_plan = nullptr;  // why the row pointer / row plan was not built, when it was skipped unchecked
 };
 
 static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr, const int32_t *indices,
@@ -684,7 +685,15 @@ int fg_sddmm_coo_mh_f32(int64_t nnz, const int32_t *row, const int32_t *col, con
 // cuts every row into column blocks (only when each row's column ids ascend; otherwise whole rows).
 // Leaves p->rows null for any other list.
 static int build_row_runs(fg_sddmm_plan *p, int32_t num_col_partitions) {
-  if (fg::config().sddmm_rows == 0 || p->nnz == 0 || p->n_rows >= 0x7fffffffLL || p->nnz > 0x7fffffffLL) return FG_OK;
+  if (p->nnz == 0) return FG_OK;
+  if (fg::config().sddmm_rows == 0) {
+    p->no_row_plan = "the plan was created with sddmm.rows = 0, which skips the row pointer";
+    return FG_OK;
+  }
+  if (p->n_rows >= 0x7fffffffLL || p->nnz > 0x7fffffffLL) {
+    p->no_row_plan = "the row plan needs n_rows and nnz below 2^31";
+    return FG_OK;
+  }
   int *flag = nullptr;
   int bad = 0;
   FG_HIP_TRY(hipMalloc(&flag, sizeof(int)));
@@ -919,6 +928,8 @@ int fg_sddmm_softmax_plan_f32(const fg_sddmm_plan *plan, const float *src, const
   if (plan->nnz == 0) return FG_OK;
   if (int rc = check_device(plan->device)) return rc;
   if (!src || !dst || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
+  if (plan->no_row_plan)  // the list's order was never looked at: do not blame it
+    return fg::fail(FG_EUNSUPPORTED, "edge softmax needs the plan's row pointer: %s", plan->no_row_plan);
   if (!plan->indptr || !plan->rows || !plan->input_row_sorted)
     return fg::fail(FG_EUNSUPPORTED, "edge softmax needs a row-sorted edge list (each destination row's edges consecutive)");
   hipStream_t st = static_cast<hipStream_t>(stream);

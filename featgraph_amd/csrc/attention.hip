@@ -135,15 +135,16 @@ __global__ __launch_bounds__(kBlockThreads) void attention_kernel(const AttnArgs
           top = fmaxf(top, s[u]);
         }
         // the first neighbour of a batch always exists, so `top` is a score: exp(-inf - top) = 0 clears the
-        // empty state and the neighbours past the row's end alike
-        const float keep = expf(m[k] - top);
+        // empty state and the neighbours past the row's end alike.  A score can itself be -inf (infinite
+        // features): such a neighbour, like an empty state, weighs 0 rather than exp(-inf - -inf) = NaN
+        const float keep = m[k] == -__builtin_inff() ? 0.0f : expf(m[k] - top);
         m[k] = top;
         l[k] *= keep;
 #pragma unroll
         for (int q = 0; q < VW; ++q) acc[k].v[q] *= keep;
 #pragma unroll
         for (int u = 0; u < CH; ++u) {
-          const float w = expf(s[u] - top);
+          const float w = s[u] == -__builtin_inff() ? 0.0f : expf(s[u] - top);
           l[k] += w;
 #pragma unroll
           for (int q = 0; q < VW; ++q)

@@ -33,6 +33,9 @@ struct MaxSum {
 };
 
 __device__ __forceinline__ void absorb(MaxSum &s, float x) {
+  // a masked edge (score -inf) adds nothing, whichever position it has: without this a -inf that comes before
+  // the row's first finite score would compute exp(-inf - -inf) = NaN
+  if (x == -__builtin_inff()) return;
   if (x > s.m) {
     s.l = s.l * expf(s.m - x) + 1.0f;  // exp(-inf) = 0 covers the first score
     s.m = x;

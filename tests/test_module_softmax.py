@@ -40,6 +40,66 @@ def test_edge_softmax_with_empty_rows_single_edges_and_large_scores():
     np.testing.assert_allclose(out, ref.edge_softmax(indptr, scores), rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("H", [2, 1])
+def test_edge_softmax_masked_edges(H):
+    """Scores of -inf (masked edges) weigh exactly 0 wherever they stand in the row, also before its first finite
+    score; a row and head with nothing else is NaN, as in the checker and in scipy.special.softmax."""
+    from test_oracle import _masked_scores
+    indptr, scores = _masked_scores()
+    scores = np.ascontiguousarray(scores[:, :H])
+    n, nnz = len(indptr) - 1, int(indptr[-1])
+    adj = scipy.sparse.csr_matrix((np.ones(nnz, np.float32), np.zeros(nnz, np.int32), indptr), shape=(n, 1))
+    out = _softmax_module(adj, scores)
+    with np.errstate(invalid="ignore"):
+        want = ref.edge_softmax(indptr, scores)
+    np.testing.assert_allclose(out, want, rtol=RTOL, atol=ATOL, equal_nan=True)
+    assert out[0, 0] == 0 and out[103, 0] == 0 and out[210, 0] == 0 and np.isfinite(out[:, 0]).all()
+    if H == 2:
+        assert np.isnan(out[140:210, 1]).all()
+
+
+def test_attention_with_infinite_scores():
+    """Neighbours whose key row holds -inf in one head get a score of -inf there: weight 0 for them, the other
+    neighbours unaffected, whichever position they have in the row (first of the first batch included)."""
+    from featgraph_amd.module import MultiHeadAttentionhip
+    rng = np.random.default_rng(31)
+    H, D, n = 8, 16, 300
+    adj = scipy.sparse.random(n, n, density=0.1, format="csr", random_state=rng, dtype=np.float32)
+    adj.sort_indices()
+    key = rng.standard_normal((n, H, D), dtype=np.float32) * np.float32(0.3)
+    value = rng.standard_normal((n, H, D), dtype=np.float32)
+    query = np.abs(rng.standard_normal((n, H, D), dtype=np.float32)) + np.float32(0.1)   # positive: -inf * q = -inf
+    masked = np.unique(np.concatenate([adj.indices[adj.indptr[:-1][np.diff(adj.indptr) > 0]][:40],   # first neighbours
+                                       rng.integers(0, n, 20)]))
+    key[masked, 3, 0] = -np.inf
+    module = MultiHeadAttentionhip(adj)
+    ins = [key, query, value]
+    module.build([placeholder(x.shape) for x in ins], {}, {})
+    out = module.run([nd.array(x, module.ctx) for x in ins]).asnumpy()
+    with np.errstate(invalid="ignore"):
+        want = ref.attention_mh(adj.indptr, adj.indices, key, query, value)
+    np.testing.assert_allclose(out, want, rtol=1e-4, atol=1e-5, equal_nan=True)
+    # NaN only where the checker has it (rows whose every neighbour is masked in head 3), never in another head
+    assert np.isfinite(out[:, [0, 1, 2, 4, 5, 6, 7]]).all()
+    assert np.isfinite(out[:, 3]).any()
+
+
+def test_fused_operator_names_a_skipped_row_plan():
+    """With sddmm.rows = 0 at plan creation the row pointer is never built: the error must say so instead of
+    blaming the (sorted) edge list."""
+    adj = datasets.config_graph("c1")
+    try:
+        _lib.config_set("sddmm.rows", 0)
+        with pytest.raises((ValueError, RuntimeError)) as err:
+            module = MultiHeadSDDMMSoftmaxhip(adj)
+            module.build([placeholder((adj.shape[1], 8, 16)), placeholder((adj.shape[0], 8, 16))], {}, {})
+            z = np.zeros((adj.shape[0], 8, 16), np.float32)
+            module.run([nd.array(z, module.ctx), nd.array(z, module.ctx)])
+    finally:
+        _lib.config_set("sddmm.rows", -1)
+    assert "sddmm.rows" in str(err.value)
+
+
 def test_edge_softmax_in_place_through_the_c_abi():
     import torch
     adj = datasets.config_graph("c4-mini")

@@ -347,6 +347,34 @@ def test_edge_softmax_against_scipy_and_its_invariants():
     np.testing.assert_allclose(uniform, (1.0 / deg)[:, None].repeat(H, 1), rtol=1e-6)
 
 
+def _masked_scores():
+    """Three rows of 70 edges (longer than one wave step), one head-pair: -inf first, -inf in the middle, all -inf."""
+    indptr = np.array([0, 70, 140, 210, 213], dtype=np.int32)
+    scores = (np.random.default_rng(23).standard_normal((213, 2)) * 3).astype(np.float32)
+    scores[0, :] = -np.inf            # before the row's first finite score
+    scores[1, 0] = -np.inf
+    scores[70 + 33, :] = -np.inf      # between finite scores
+    scores[140:210, 1] = -np.inf      # every score of (row 2, head 1)
+    scores[210, 0] = -np.inf          # a short row whose first score is masked
+    return indptr, scores
+
+
+def test_edge_softmax_masked_edges_against_scipy():
+    """A score of -inf is a masked edge: weight exactly 0, the others as if it were absent (scipy.special.softmax);
+    a row and head with nothing but -inf is 0/0 = NaN there, and in the checker too."""
+    import scipy.special
+    indptr, scores = _masked_scores()
+    with np.errstate(invalid="ignore"):
+        out = ref.edge_softmax(indptr, scores)
+        for r in range(4):
+            sl = slice(indptr[r], indptr[r + 1])
+            want = scipy.special.softmax(scores[sl].astype(np.float64), axis=0)
+            np.testing.assert_allclose(out[sl], want, rtol=1e-6, equal_nan=True)
+    assert out[0, 0] == 0 and out[0, 1] == 0 and out[1, 0] == 0 and out[103, 0] == 0 and out[210, 0] == 0
+    assert np.isnan(out[140:210, 1]).all() and np.isfinite(out[140:210, 0]).all()
+    assert abs(out[:70, 0].astype(np.float64).sum() - 1) < 1e-6
+
+
 def test_attention_against_dense_masked_softmax():
     """The composed checker against the textbook dense form: softmax over a row's stored entries of Q K^T, times V
     (float64 einsum on a matrix small enough to densify), with separate and with shared key / value."""
