@@ -51,6 +51,9 @@ struct fg_spmm_plan {
   // When the library sizes the blocks it may cut each block of the default width into `split` equal ones, so
   // that a kernel can take 1 .. split neighbouring blocks per pass; split_used is 1 when the caller sized them.
   int32_t split = 1, split_used = 1;
+  // the library's own blocks come in a multiple of eight default-width passes (when there are seven or more), so
+  // that passes pinned to the eight dies keep every die busy in every round
+  bool xcd_round = false;
   int32_t requested_partitions;  // 0: library decides; 1: no column blocks; P > 1: P blocks, as the caller asked
   bool force_blocks;             // the caller's P > 1: use the blocks at every feature length
   // what the bounds table is built from: block width (0: default), blocks on / off / automatic (1 / 0 / -1),
@@ -86,7 +89,7 @@ struct fg_sddmm_plan {
 static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr, const int32_t *indices,
                            int32_t num_col_partitions, int32_t want_block_cols, int32_t default_block_cols,
                            int32_t split, int want_blocked, double min_per_segment, bool with_multi,
-                           fg_spmm_plan **plan);
+                           bool xcd_round, fg_spmm_plan **plan);
 
 namespace {
 
@@ -367,6 +370,7 @@ int build_bounds(fg_spmm_plan *p) {
   // the library's own blocks: as many as the default width asks for (times the split), all of the same width
   p->split_used = 1;
   if (P <= 1 && p->want_block_cols <= 0 && n_blocks > 1) {
+    if (p->xcd_round && n_blocks >= fg::kXcds - 1) n_blocks = (n_blocks + fg::kXcds - 1) / fg::kXcds * fg::kXcds;
     p->split_used = std::max(1, p->split);
     n_blocks *= p->split_used;
     block_cols = (p->n_cols + n_blocks - 1) / n_blocks;
@@ -448,6 +452,8 @@ int *config_slot(const char *key) {
   if (!strcmp(key, "sddmm.rows_wide")) return &c.sddmm_rows_wide;
   if (!strcmp(key, "sddmm.sorted_copy")) return &c.sddmm_sorted_copy;
   if (!strcmp(key, "sddmm.regroup")) return &c.sddmm_regroup;
+  if (!strcmp(key, "sddmm.xcd")) return &c.sddmm_xcd;
+  if (!strcmp(key, "spmm.xcd")) return &c.spmm_xcd;
   if (!strcmp(key, "attention.blocks")) return &c.attention_blocks;
   return nullptr;
 }
@@ -490,7 +496,7 @@ int fg_spmm_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32
 int fg_spmm_plan_create_partitioned(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr,
                                     const int32_t *indices, int32_t num_col_partitions, fg_spmm_plan **plan) {
   return row_plan_create(n_rows, n_cols, nnz, indptr, indices, num_col_partitions, fg::config().spmm_block_cols,
-                         kSpmmBlockCols, 1, fg::config().spmm_blocked, 8.0, true, plan);
+                         kSpmmBlockCols, 1, fg::config().spmm_blocked, 8.0, true, false, plan);
 }
 
 // want_block_cols / want_blocked / min_per_segment: see fg_spmm_plan; with_multi: also build the records of the
@@ -498,7 +504,7 @@ int fg_spmm_plan_create_partitioned(int64_t n_rows, int64_t n_cols, int64_t nnz,
 static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *indptr, const int32_t *indices,
                            int32_t num_col_partitions, int32_t want_block_cols, int32_t default_block_cols,
                            int32_t split, int want_blocked, double min_per_segment, bool with_multi,
-                           fg_spmm_plan **plan) {
+                           bool xcd_round, fg_spmm_plan **plan) {
   if (!plan) return fg::fail(FG_EINVAL, "plan output pointer is null");
   *plan = nullptr;
   if (num_col_partitions < 0)
@@ -550,6 +556,7 @@ static int row_plan_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const in
   p->want_block_cols = want_block_cols;
   p->default_block_cols = default_block_cols;
   p->split = split;
+  p->xcd_round = xcd_round;
   p->want_blocked = want_blocked;
   p->min_per_segment = min_per_segment;
   p->max_degree = max_degree;
@@ -731,7 +738,7 @@ static int build_row_runs(fg_sddmm_plan *p, int32_t num_col_partitions) {
   // work, so blocks need 8 edges per run on average (sparser lists keep whole rows and take the edge-list path)
   if (int rc = row_plan_create(p->n_rows, p->n_cols, p->nnz, p->indptr, cols_of, num_col_partitions,
                                fg::config().sddmm_block_cols, kSddmmBlockCols, kSddmmSplit, fg::config().sddmm_blocked,
-                               8.0, false, &p->rows))
+                               8.0, false, fg::config().sddmm_xcd != 0, &p->rows))
     return rc;
   if (p->sorted.col_s && !(p->rows && p->rows->seg && p->rows->n_blocks >= 2)) {
     // too thin for column blocks: the sorted copy would buy nothing over the caller's list
@@ -752,7 +759,7 @@ static int build_row_runs(fg_sddmm_plan *p, int32_t num_col_partitions) {
       fg_spmm_plan *blocked = nullptr;
       if (int rc = row_plan_create(p->n_rows, p->n_cols, p->nnz, p->indptr, p->sorted.col_s, num_col_partitions,
                                    fg::config().sddmm_block_cols, kSddmmBlockCols, kSddmmSplit,
-                                   fg::config().sddmm_blocked, 8.0, false, &blocked))
+                                   fg::config().sddmm_blocked, 8.0, false, fg::config().sddmm_xcd != 0, &blocked))
         return rc;
       if (blocked && blocked->seg && blocked->n_blocks >= 2) {
         fg_spmm_plan_destroy(p->rows);
@@ -1022,7 +1029,8 @@ int fg_config_set(const char *key, int32_t value) {
                     slot == &fg::config().sddmm_buffer_loads || slot == &fg::config().sddmm_rows ||
                     slot == &fg::config().spmm_multi || slot == &fg::config().sddmm_sorted_copy ||
                     slot == &fg::config().sddmm_regroup || slot == &fg::config().spmm_relay ||
-                    slot == &fg::config().spmm_general_multi;
+                    slot == &fg::config().spmm_general_multi || slot == &fg::config().sddmm_xcd ||
+                    slot == &fg::config().spmm_xcd;
   // flags: 0 / 1 are explicit, anything negative restores the default;
   // sizes: 0 restores the default
   *slot = flag ? (value < 0 ? -1 : (value != 0)) : std::max(value, 0);

@@ -29,9 +29,13 @@ struct Config {
   int sddmm_group = 0, sddmm_batches = 0, sddmm_blocked = -1, sddmm_block_cols = 0;
   int sddmm_fast = -1, sddmm_buffer_loads = -1, sddmm_rows = -1, sddmm_rows_blocks = 0;
   int attention_blocks = 0, sddmm_rows_wide = 0, sddmm_sorted_copy = -1, sddmm_regroup = -1, spmm_relay = -1, spmm_general_multi = -1;
+  int sddmm_xcd = -1, spmm_xcd = -1;
 };
 Config &config();
 
+// Accelerator complex dies of the part, each with its own L2; workgroups of a launch go to them round-robin by
+// their linear id (measured on MI355X: hardware XCC id == workgroup id % 8).
+constexpr int kXcds = 8;
 constexpr int kWaveSize = 64;
 constexpr int kWavesPerBlock = 4;
 constexpr int kBlockThreads = kWaveSize * kWavesPerBlock;

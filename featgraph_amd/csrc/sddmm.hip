@@ -243,8 +243,26 @@ struct RowsArgs {
   int64_t src_bytes, dst_bytes;
   int32_t n_rows, F;
   int32_t first, valid;      // the tile this launch covers
-  int32_t n_blocks, merge;   // column blocks in the table; blockIdx.y covers `merge` neighbouring ones
+  int32_t n_blocks, merge;   // column blocks in the table; a pass covers `merge` neighbouring ones
+  // Passes pinned to the dies: workgroup x of a launch runs on die x % 8, so the workgroups x % 8 == d take the
+  // passes d, d + 8, ... (blockIdx.y counts those rounds) and every die's L2 keeps the band of ITS pass while the
+  // die walks all rows, instead of all eight L2s holding copies of one band.  0: blockIdx.y is the pass.
+  int32_t xcd_passes = 0;
 };
+
+// (pass, first item, item stride) of a workgroup's wave under either numbering.
+__device__ __forceinline__ void rows_wave_place(const RowsArgs &a, int &pass, int &item, int &n_waves) {
+  const int wave = static_cast<int>(threadIdx.x >> 6);
+  if (a.xcd_passes) {
+    pass = static_cast<int>(blockIdx.y) * kXcds + static_cast<int>(blockIdx.x % kXcds);
+    item = static_cast<int>(blockIdx.x / kXcds) * kWavesPerBlock + wave;
+    n_waves = static_cast<int>(gridDim.x / kXcds) * kWavesPerBlock;
+  } else {
+    pass = static_cast<int>(blockIdx.y);
+    item = static_cast<int>(blockIdx.x) * kWavesPerBlock + wave;
+    n_waves = static_cast<int>(gridDim.x) * kWavesPerBlock;
+  }
+}
 
 // G: lanes per dot product; NT: 16-byte pieces per lane, 64 floats apart (a tile is 4 * G * NT floats; NT > 1
 // needs G = 16); R: rounds whose gathers are issued together.
@@ -255,11 +273,13 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_rows_kernel(const RowsArg
   const int lane = threadIdx.x & (kWaveSize - 1);
   const int gl = lane & (G - 1);
   const int g = lane / G;
-  const int n_waves = gridDim.x * kWavesPerBlock;
   const int n = a.n_rows;
-  int item = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)));
-  const int32_t *const seg_lo = a.seg + static_cast<int64_t>(blockIdx.y) * a.merge * n;
-  const int32_t *const seg_hi = a.seg + static_cast<int64_t>(min((blockIdx.y + 1) * a.merge, a.n_blocks)) * n;
+  int pass, item, n_waves;
+  rows_wave_place(a, pass, item, n_waves);
+  item = __builtin_amdgcn_readfirstlane(item);
+  if (pass * a.merge >= a.n_blocks) return;
+  const int32_t *const seg_lo = a.seg + static_cast<int64_t>(pass) * a.merge * n;
+  const int32_t *const seg_hi = a.seg + static_cast<int64_t>(min((pass + 1) * a.merge, a.n_blocks)) * n;
   const VertexRows<BUF> src(a.src, a.src_bytes), dst(a.dst, a.dst_bytes);
   const uint32_t row_bytes = static_cast<uint32_t>(a.F) * 4u;
   // piece k of this lane covers floats first + 64 k + 4 gl ..; lanes past the tile's end re-read its last
@@ -400,11 +420,13 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_rows_elementwise_kernel(c
   const int lane = threadIdx.x & (kWaveSize - 1);
   const int gl = lane & (G - 1);
   const int g = lane / G;
-  const int n_waves = gridDim.x * kWavesPerBlock;
   const int n = a.n_rows;
-  int item = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)));
-  const int32_t *const seg_lo = a.seg + static_cast<int64_t>(blockIdx.y) * a.merge * n;
-  const int32_t *const seg_hi = a.seg + static_cast<int64_t>(min((blockIdx.y + 1) * a.merge, a.n_blocks)) * n;
+  int pass, item, n_waves;
+  rows_wave_place(a, pass, item, n_waves);
+  item = __builtin_amdgcn_readfirstlane(item);
+  if (pass * a.merge >= a.n_blocks) return;
+  const int32_t *const seg_lo = a.seg + static_cast<int64_t>(pass) * a.merge * n;
+  const int32_t *const seg_hi = a.seg + static_cast<int64_t>(min((pass + 1) * a.merge, a.n_blocks)) * n;
   const VertexRows<BUF> src(a.src, a.src_bytes), dst(a.dst, a.dst_bytes);
   const uint32_t row_bytes = static_cast<uint32_t>(a.F) * 4u;
   const bool kok = gl * 4 < a.valid;  // lanes past the tile's end re-read its last four floats and store nothing
@@ -620,6 +642,17 @@ int sddmm_rows_tile(int32_t F, int max_wide) {
   return 64;
 }
 
+// Grid of a row-run launch over `passes` passes with `blocks` workgroups each.  With eight passes or more the
+// passes are pinned to the dies (RowsArgs::xcd_passes): grid.x = 8 * blocks, grid.y = rounds of eight passes;
+// workgroups are dispatched x-fastest and 8 divides grid.x, so workgroup (x, y) runs on die x % 8.
+static dim3 rows_grid(RowsArgs &a, int64_t blocks, int passes) {
+  const int want = config().sddmm_xcd;
+  a.xcd_passes = (want != 0 && passes >= kXcds) ? 1 : 0;
+  if (a.xcd_passes)
+    return dim3(static_cast<unsigned>(blocks * kXcds), static_cast<unsigned>((passes + kXcds - 1) / kXcds));
+  return dim3(static_cast<unsigned>(blocks), static_cast<unsigned>(passes));
+}
+
 int sddmm_rows_launch(const int32_t *seg, const int32_t *row_order, int32_t n_rows, int32_t n_blocks, int32_t merge64,
                       int max_wide, const int32_t *col, const float *src, const float *dst, float *out,
                       int64_t src_bytes, int64_t dst_bytes, int32_t F, hipStream_t stream) {
@@ -649,7 +682,7 @@ int sddmm_rows_launch(const int32_t *seg, const int32_t *row_order, int32_t n_ro
     a.merge = merge;
     a.first = first;
     a.valid = std::min(F - first, tile);
-    const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>((n_blocks + merge - 1) / merge));
+    const dim3 grid = rows_grid(a, blocks, (n_blocks + merge - 1) / merge);
     const bool acc = first > 0;
     if (tile == 16)
       rows_dispatch<4, 1>(a, acc, buf, grid, stream);
@@ -706,7 +739,7 @@ int sddmm_rows_elementwise_launch(const int32_t *seg, const int32_t *row_order, 
     a.merge = std::max(1, std::min(merge64 * (64 / tile), n_blocks));
     a.first = first;
     a.valid = std::min(F - first, tile);
-    const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>((n_blocks + a.merge - 1) / a.merge));
+    const dim3 grid = rows_grid(a, blocks, (n_blocks + a.merge - 1) / a.merge);
     switch (op) {
       case FG_EDGE_ADD: rows_elementwise_dispatch<FG_EDGE_ADD>(a, tile, buf, grid, stream); break;
       case FG_EDGE_SUB: rows_elementwise_dispatch<FG_EDGE_SUB>(a, tile, buf, grid, stream); break;

@@ -407,6 +407,12 @@ FG_API int64_t fg_probe_store_rows_f32(float *out, int64_t n_out_rows, int32_t r
  * works on a sorted copy, read at plan creation; default 1), "sddmm.regroup"
  * (0/1: whether such a plan returns the results through two block-local
  * permutations or one gather, read at plan creation; default 1),
+ * "sddmm.xcd" (0/1: whether the passes of the row-run kernel are pinned to the
+ * part's eight dies -- workgroup x of a launch runs on die x % 8, so the
+ * workgroups x % 8 == d take the passes d, d + 8, ... and each die's L2 keeps
+ * the band of its own pass -- and whether the library's own blocks come in a
+ * multiple of eight passes; read at plan creation and at launch; default 1;
+ * same result bits either way),
  * "attention.blocks" (grid size of the fused attention kernel; by default one
  * vertex row per wave when a row is 1 KB or more, else 65536 workgroups that
  * walk the rows).  Value 0 restores the default of a size; for the 0/1 flags a

@@ -33,7 +33,8 @@ def config_guard():
     _lib.config_set("sddmm.block_cols", 0)
     _lib.config_set("sddmm.rows_blocks", 0)
     _lib.config_set("sddmm.rows_wide", 0)
-    for key in ("sddmm.blocked", "sddmm.fast", "sddmm.buffer_loads", "sddmm.rows", "sddmm.sorted_copy", "sddmm.regroup"):
+    for key in ("sddmm.blocked", "sddmm.fast", "sddmm.buffer_loads", "sddmm.rows", "sddmm.sorted_copy", "sddmm.regroup",
+                "sddmm.xcd"):
         _lib.config_set(key, -1)
 
 
@@ -309,6 +310,21 @@ def test_which_lists_take_the_row_run_kernel(config_guard):
     # 30 floats or several heads: neither blocked kernel applies
     src30, dst30 = datasets.sddmm_operands(coo, 30)
     assert "row runs" not in _describe(VanillaSDDMMhip(coo), src30, dst30)
+
+
+@pytest.mark.parametrize("F,block_cols", [(64, 500), (32, 300), (256, 700), (64, 1000)])
+def test_passes_pinned_to_the_dies_change_no_bit(config_guard, F, block_cols):
+    """With eight passes or more the row-run kernel numbers its workgroups so that each die keeps to its own
+    passes (12, 20, 9 and 6 passes here: whole rounds of eight, a partial last round, and too few to pin): the
+    same runs by the same code, so the results equal those of the pass-by-pass numbering bit for bit."""
+    coo = datasets.config_graph("c2-mini").tocoo()
+    src, dst = datasets.sddmm_operands(coo, F)
+    _lib.config_set("sddmm.block_cols", block_cols)
+    _lib.config_set("sddmm.xcd", 1)
+    pinned = _run_sddmm(coo, src, dst)
+    _lib.config_set("sddmm.xcd", 0)
+    assert np.array_equal(_run_sddmm(coo, src, dst), pinned)
+    np.testing.assert_allclose(pinned, ref.sddmm_f64(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
 
 
 @pytest.mark.parametrize("regroup", [1, 0])
