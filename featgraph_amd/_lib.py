@@ -22,6 +22,10 @@ SIGNATURES = {
     "fg_spmm_csr_f32": (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _p]),
     "fg_spmm_csr_noalloc_f32": (ctypes.c_int, [_i64, _i64, _i64, _p, _p, _p, _p, _p, _i32, _p]),
     "fg_spmm_csr_general_f32": (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _i32, _p]),
+    "fg_spmm_csr_mh_general_f32": (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _i32, _i32, _p]),
+    "fg_edge_softmax_backward_csr_f32": (ctypes.c_int, [_i64, _p, _p, _p, _p, _i32, _p]),
+    "fg_permute_rows_f32": (ctypes.c_int, [_i64, _i32, _p, _p, _p, _p]),
+    "fg_add_f32": (ctypes.c_int, [_i64, _p, _p, _p, _p]),
     "fg_sddmm_coo_general_f32": (ctypes.c_int, [_i64, _p, _p, _p, _p, _p, _i32, _i32, _p]),
     "fg_spmm_csr_mh_f32": (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _i32, _p]),
     "fg_sddmm_coo_f32": (ctypes.c_int, [_i64, _p, _p, _p, _p, _p, _i32, _p]),

@@ -14,7 +14,7 @@ CSRC = os.path.join(_PKG, "csrc")
 LIB_DIR = os.path.join(_PKG, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libfeatgraph_hip.so")
 SOURCES = ("api.hip", "spmm.hip", "spmm_multi.hip", "spmm_multi_general_mul.hip", "spmm_multi_general_add.hip",
-           "spmm_multi_general_sub.hip", "spmm_multi_general_div.hip", "spmm_multi_general_copy_u.hip", "sddmm.hip", "sddmm_blocked.hip", "sddmm_sorted.hip", "noalloc.hip", "probe.hip", "general.hip", "softmax.hip", "attention.hip")
+           "spmm_multi_general_sub.hip", "spmm_multi_general_div.hip", "spmm_multi_general_copy_u.hip", "sddmm.hip", "sddmm_blocked.hip", "sddmm_sorted.hip", "noalloc.hip", "probe.hip", "general.hip", "softmax.hip", "attention.hip", "backward.hip")
 
 # -ffp-contract=off: the SpMM kernels must round the product and the sum
 # separately (fused multiply-adds are written explicitly where wanted).

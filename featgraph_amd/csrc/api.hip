@@ -664,6 +664,49 @@ int fg_spmm_csr_general_f32(const fg_spmm_plan *plan, const float *feat, const f
                                  static_cast<int32_t>(plan->n_rows), F, msg, reduce, st);
 }
 
+int fg_spmm_csr_mh_general_f32(const fg_spmm_plan *plan, const float *feat, const float *w, float *out, int32_t H,
+                               int32_t D, int32_t msg, int32_t reduce, void *stream) {
+  if (H == 1) return fg_spmm_csr_general_f32(plan, feat, w, out, D, msg, reduce, stream);
+  if (!plan) return fg::fail(FG_EINVAL, "plan is null");
+  if (int rc = check_heads(H, D)) return rc;
+  if (int rc = check_device(plan->device)) return rc;
+  if (msg < FG_MSG_MUL || msg > FG_MSG_COPY_U) return fg::fail(FG_EINVAL, "msg = %d is not an FG_MSG_* code", msg);
+  if (reduce < FG_REDUCE_SUM || reduce > FG_REDUCE_MEAN)
+    return fg::fail(FG_EINVAL, "reduce = %d is not an FG_REDUCE_* code", reduce);
+  if (plan->n_rows > 0 && !out) return fg::fail(FG_EINVAL, "out is null");
+  if (plan->nnz > 0 && (!feat || (!w && msg != FG_MSG_COPY_U)))
+    return fg::fail(FG_EINVAL, "feat or edge weights are null");
+  if (plan->n_rows == 0) return FG_OK;
+  return fg::spmm_general_mh_launch(plan->row_order, plan->seg, plan->n_blocks, plan->indices, w, feat, out,
+                                    static_cast<int32_t>(plan->n_rows), H, D, msg, reduce,
+                                    static_cast<hipStream_t>(stream));
+}
+
+int fg_edge_softmax_backward_csr_f32(int64_t n_rows, const int32_t *indptr, const float *weights, const float *grad,
+                                     float *out, int32_t H, void *stream) {
+  if (n_rows < 0 || n_rows >= 0x7fffffffLL) return fg::fail(FG_EINVAL, "n_rows = %lld is out of range", (long long)n_rows);
+  if (H < 1 || H > (1 << 20)) return fg::fail(FG_EINVAL, "H = %d is out of range", H);
+  if (n_rows == 0) return FG_OK;
+  if (!indptr || !weights || !grad || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
+  return fg::edge_softmax_backward_launch(indptr, weights, grad, out, static_cast<int32_t>(n_rows), H,
+                                          static_cast<hipStream_t>(stream));
+}
+
+int fg_permute_rows_f32(int64_t n, int32_t width, const int32_t *perm, const float *in, float *out, void *stream) {
+  if (n < 0) return fg::fail(FG_EINVAL, "n = %lld is negative", (long long)n);
+  if (width < 1 || width > (1 << 20)) return fg::fail(FG_EINVAL, "width = %d is out of range", width);
+  if (n == 0) return FG_OK;
+  if (!perm || !in || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
+  return fg::permute_rows_launch(perm, in, out, n, width, static_cast<hipStream_t>(stream));
+}
+
+int fg_add_f32(int64_t n, const float *a, const float *b, float *out, void *stream) {
+  if (n < 0) return fg::fail(FG_EINVAL, "n = %lld is negative", (long long)n);
+  if (n == 0) return FG_OK;
+  if (!a || !b || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
+  return fg::add_launch(a, b, out, n, static_cast<hipStream_t>(stream));
+}
+
 int fg_sddmm_coo_general_f32(int64_t nnz, const int32_t *row, const int32_t *col, const float *src, const float *dst,
                              float *out, int32_t F, int32_t edge_op, void *stream) {
   if (edge_op == FG_EDGE_DOT) return fg_sddmm_coo_f32(nnz, row, col, src, dst, out, F, stream);

@@ -196,6 +196,10 @@ int sddmm_rows_elementwise_launch(const int32_t *seg, const int32_t *row_order, 
 int spmm_general_launch(const int32_t *row_order, const int32_t *seg, int32_t n_blocks, const int32_t *indices,
                         const float *vals, const float *feat, float *out, int32_t n_rows, int32_t F, int msg,
                         int reduce, hipStream_t stream);
+// ... with H heads of D floats and per-edge per-head values vals [nnz, H]
+int spmm_general_mh_launch(const int32_t *row_order, const int32_t *seg, int32_t n_blocks, const int32_t *indices,
+                           const float *vals, const float *feat, float *out, int32_t n_rows, int32_t H, int32_t D,
+                           int msg, int reduce, hipStream_t stream);
 // out[r, :] /= degree of row r (rows without nonzeros stay 0): the last step of the mean over a sum
 int spmm_mean_finish_launch(const int32_t *indptr, float *out, int32_t n_rows, int32_t F, hipStream_t stream);
 int sddmm_elementwise_launch(const int32_t *row, const int32_t *col, const float *src, const float *dst, float *out,
@@ -207,6 +211,13 @@ int edge_softmax_launch(const int32_t *indptr, const float *scores, float *out, 
 bool sddmm_softmax_fused_applies(const float *src, const float *dst, int32_t H, int32_t D);
 int sddmm_softmax_launch(const int32_t *row_order, const int32_t *indptr, const int32_t *indices, const float *src,
                          const float *dst, float *out, int32_t n_rows, int32_t H, int32_t D, hipStream_t stream);
+
+// Pieces of the multi-head backward (backward.hip): gradient of the edge softmax, rows gathered through a
+// permutation, elementwise sum.
+int edge_softmax_backward_launch(const int32_t *indptr, const float *weights, const float *grad, float *out,
+                                 int32_t n_rows, int32_t H, hipStream_t stream);
+int permute_rows_launch(const int32_t *perm, const float *in, float *out, int64_t n, int32_t width, hipStream_t stream);
+int add_launch(const float *a, const float *b, float *out, int64_t n, hipStream_t stream);
 
 // Multi-head SDDMM, edge softmax and multi-head SpMM as one kernel (attention.hip).
 bool attention_fused_applies(const float *key, const float *query, const float *value, const float *out, int32_t H,

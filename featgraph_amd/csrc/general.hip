@@ -53,9 +53,12 @@ struct GeneralArgs {
   const float *feat;
   float *out;
   int32_t n_rows, F, n_tiles;
+  int32_t H = 1, D = 0;      // multi-head: vals is [nnz, H] and float f of a row belongs to head f / D
 };
 
-template <int VEC, int LPR, int MSG, int RED>
+// MH: per-edge per-head values; a lane's VEC floats lie inside one head (D is a multiple of VEC), and the lane
+// reads its head's value of every nonzero itself.
+template <int VEC, int LPR, int MSG, int RED, bool MH>
 __global__ __launch_bounds__(kBlockThreads) void spmm_general_kernel(const GeneralArgs a) {
   constexpr int RPW = kWaveSize / LPR;
   constexpr int TW = VEC * LPR;
@@ -74,6 +77,8 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_general_kernel(const Gener
   const int64_t F = a.F;
   const float *fp = a.feat + (fok ? f0 : a.F - VEC);
   float *op = a.out + static_cast<int64_t>(row) * F + f0;
+  const int head = MH ? (fok ? f0 : a.F - VEC) / a.D : 0;
+  const int64_t H = a.H;
   // A pass continues the fold where the pass before it stopped: the value it left in Out.  The pass that holds
   // the row's first nonzero starts afresh (sum: from +0; max / min: with the first message itself, as the
   // reference order of evaluation has it), and a pass without nonzeros of the row leaves Out alone.
@@ -104,7 +109,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_general_kernel(const Gener
   float next_val = 1.0f;
   if (sl < end - first) {
     next_col = a.indices[first + sl];
-    if (MSG != FG_MSG_COPY_U) next_val = a.vals[first + sl];
+    if (!MH && MSG != FG_MSG_COPY_U) next_val = a.vals[first + sl];
   }
   for (int e = first; e < end; e += LPR) {
     const int n = min(LPR, end - e);
@@ -114,7 +119,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_general_kernel(const Gener
     next_val = 1.0f;
     if (sl < end - (e + LPR)) {
       next_col = a.indices[e + LPR + sl];
-      if (MSG != FG_MSG_COPY_U) next_val = a.vals[e + LPR + sl];
+      if (!MH && MSG != FG_MSG_COPY_U) next_val = a.vals[e + LPR + sl];
     }
     for (int j = 0; j < n; j += U) {
       float x[U][VEC];
@@ -123,7 +128,12 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_general_kernel(const Gener
       for (int u = 0; u < U; ++u) {
         const int from = ((lane & ~(LPR - 1)) | ((j + u) & (LPR - 1))) << 2;
         const int c = __builtin_amdgcn_ds_bpermute(from, my_col);  // slots past n hold column 0: valid, unused
-        v[u] = __int_as_float(__builtin_amdgcn_ds_bpermute(from, __float_as_int(my_val)));
+        if constexpr (MH) {
+          v[u] = 1.0f;
+          if (MSG != FG_MSG_COPY_U && j + u < n) v[u] = a.vals[static_cast<int64_t>(e + j + u) * H + head];
+        } else {
+          v[u] = __int_as_float(__builtin_amdgcn_ds_bpermute(from, __float_as_int(my_val)));
+        }
         const float *p = fp + static_cast<int64_t>(c) * F;
         if constexpr (VEC == 4) {
           const float4 q = *reinterpret_cast<const float4 *>(p);
@@ -156,13 +166,13 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_general_kernel(const Gener
     *op = acc[0];
 }
 
-template <int VEC, int LPR, int MSG, int RED>
+template <int VEC, int LPR, int MSG, int RED, bool MH>
 int launch_general(const GeneralArgs &a, hipStream_t stream) {
   constexpr int RPW = kWaveSize / LPR;
   const int64_t slots = static_cast<int64_t>(a.n_tiles) * a.n_rows;
   const int64_t blocks = ((slots + RPW - 1) / RPW + kWavesPerBlock - 1) / kWavesPerBlock;
   if (blocks > 0x7fffffffLL) return fail(FG_EUNSUPPORTED, "generalised SpMM launch needs %lld blocks", (long long)blocks);
-  spmm_general_kernel<VEC, LPR, MSG, RED><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlockThreads), 0, stream>>>(a);
+  spmm_general_kernel<VEC, LPR, MSG, RED, MH><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlockThreads), 0, stream>>>(a);
   FG_HIP_TRY(hipGetLastError());
   return FG_OK;
 }
@@ -170,8 +180,12 @@ int launch_general(const GeneralArgs &a, hipStream_t stream) {
 template <int MSG, int RED>
 int dispatch_shape(GeneralArgs a, bool vec4, hipStream_t stream) {
   a.n_tiles = (a.F + 63) / 64;  // both shapes cover 64 floats per slot
-  if (vec4) return launch_general<4, 16, MSG, RED>(a, stream);
-  return launch_general<1, 64, MSG, RED>(a, stream);
+  if (a.H > 1) {
+    if (vec4) return launch_general<4, 16, MSG, RED, true>(a, stream);
+    return launch_general<1, 64, MSG, RED, true>(a, stream);
+  }
+  if (vec4) return launch_general<4, 16, MSG, RED, false>(a, stream);
+  return launch_general<1, 64, MSG, RED, false>(a, stream);
 }
 
 template <int MSG>
@@ -257,6 +271,14 @@ static int general_pass(GeneralArgs a, bool vec4, int msg, int reduce, hipStream
 int spmm_general_launch(const int32_t *row_order, const int32_t *seg, int32_t n_blocks, const int32_t *indices,
                         const float *vals, const float *feat, float *out, int32_t n_rows, int32_t F, int msg,
                         int reduce, hipStream_t stream) {
+  return spmm_general_mh_launch(row_order, seg, n_blocks, indices, vals, feat, out, n_rows, 1, F, msg, reduce, stream);
+}
+
+// H heads of D floats: vals is [nnz, H]; H == 1 is the single-head operator.
+int spmm_general_mh_launch(const int32_t *row_order, const int32_t *seg, int32_t n_blocks, const int32_t *indices,
+                           const float *vals, const float *feat, float *out, int32_t n_rows, int32_t H, int32_t D,
+                           int msg, int reduce, hipStream_t stream) {
+  const int32_t F = H * D;
   if (n_rows == 0) return FG_OK;
   GeneralArgs a;
   a.row_order = row_order;
@@ -268,8 +290,11 @@ int spmm_general_launch(const int32_t *row_order, const int32_t *seg, int32_t n_
   a.out = out;
   a.n_rows = n_rows;
   a.F = F;
+  a.H = H;
+  a.D = D;
   a.n_tiles = 1;
-  const bool vec4 = F % 4 == 0 && aligned_to(feat, 16) && aligned_to(out, 16);
+  // four floats per lane must lie inside one head
+  const bool vec4 = D % 4 == 0 && aligned_to(feat, 16) && aligned_to(out, 16);
   const int passes = config().spmm_blocked == 0 ? 1 : std::max(1, n_blocks);
   for (int b = 0; b < passes; ++b) {
     a.seg_lo = passes == 1 ? a.row_lo : seg + static_cast<int64_t>(b) * n_rows;

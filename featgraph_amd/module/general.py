@@ -64,6 +64,53 @@ class GeneralizedSpMMhip(SpMMbase):
             MSG_OPS[self._msg], REDUCE_OPS[self._reduce], C.current_stream_handle(self._ctx)))
 
 
+class MultiHeadGeneralizedSpMMhip(SpMMbase):
+    """Out[r, h, :] = reduce over the row's nonzeros e of msg(SrcFeat[indices[e], h, :], EdgeWeight[e, h]): the
+    generalised operator with per-edge per-head values (max / mean aggregation of a multi-head layer).
+
+    build([SrcFeat (num_cols, H, D), EdgeWeight (nnz, H)], ...), run([feat, weight]); msg / reduce as for
+    GeneralizedSpMMhip.  ('mul', 'sum') is MultiHeadSpMMhip bit for bit.  The CSR values of the matrix are not used.
+    """
+
+    _input_names = ("SrcFeat", "EdgeWeight")
+
+    def __init__(self, adj_scipy, msg="mul", reduce="sum", num_col_partitions=None):
+        if msg not in MSG_OPS:
+            raise ValueError("msg must be one of %s, got %r" % (sorted(MSG_OPS), msg))
+        if reduce not in REDUCE_OPS:
+            raise ValueError("reduce must be one of %s, got %r" % (sorted(REDUCE_OPS), reduce))
+        self._msg, self._reduce = msg, reduce
+        super().__init__(adj_scipy, num_col_partitions)
+
+    def _register(self):
+        self._target = "hip"
+        self._ctx = hip(0)
+
+    def _heads_and_len(self, feat_shape):
+        if len(feat_shape) != 3:
+            raise ValueError("SrcFeat must be 3-D [num_src_vertices, num_heads, head_len], got %s" % (feat_shape,))
+        return int(feat_shape[1]), int(feat_shape[2])
+
+    def _parse_build(self, input_placeholders, compute_args, schedule_args):
+        shapes, H, D, tiles = super()._parse_build(input_placeholders, compute_args, schedule_args)
+        if shapes[1] != (self._nnz, H):
+            raise ValueError("EdgeWeight must have shape (nnz, num_heads) = %s, got %s" % ((self._nnz, H), shapes[1]))
+        return shapes, H, D, tiles
+
+    def lower_to_ir(self, input_placeholders, compute_args, schedule_args):
+        _, H, D, _ = self._parse_build(input_placeholders, compute_args, schedule_args)
+        return ("spmm_csr_mh_general rows=%d cols=%d nnz=%d H=%d D=%d | msg=%s reduce=%s | kernel=row-slot, "
+                "rows=by-descending-degree, %d floats/lane, tile=64 floats x %d tiles" % (
+                    self._num_rows, self._num_cols, self._nnz, H, D, self._msg, self._reduce,
+                    4 if D % 4 == 0 else 1, (H * D + 63) // 64))
+
+    def _launch(self, tensors):
+        feat, weight = tensors
+        _lib.check(_lib.lib().fg_spmm_csr_mh_general_f32(
+            self._plan, feat.data_ptr(), weight.data_ptr(), self.out_tvm.tensor.data_ptr(), self._H, self._D,
+            MSG_OPS[self._msg], REDUCE_OPS[self._reduce], C.current_stream_handle(self._ctx)))
+
+
 class GeneralizedSDDMMhip(SDDMMbase):
     """Out[e] = <SrcFeat[col[e]], DstFeat[row[e]]> for op 'dot' (VanillaSDDMMhip), otherwise the elementwise
     edge function Out[e, :] = SrcFeat[col[e], :] op DstFeat[row[e], :] with op in {'add', 'sub', 'mul', 'div'}

@@ -166,6 +166,21 @@ FG_API int fg_spmm_csr_mh_f32(const fg_spmm_plan *plan, const float *feat, const
                        int32_t D, int32_t feat_tiles, void *stream);
 
 /*
+ * The two above combined (no counterpart in the reference): the message and
+ * reduce slots of op/vanilla_spmm.py:46-53 with a per-edge per-head value,
+ *   term(e, h, d) = msg(feat[indices[e], h, d], w[e, h])
+ *   Out[r, h, d]  = fold of the row's terms in CSR order,
+ * msg / reduce as for fg_spmm_csr_general_f32 (same folds, same treatment of
+ * rows without nonzeros, FG_REDUCE_MEAN divides by the row's degree).  feat
+ * [n_cols, H, D], w [nnz, H] (may be null for FG_MSG_COPY_U), out
+ * [n_rows, H, D].  (MUL, SUM) equals fg_spmm_csr_mh_f32 bit for bit and H = 1
+ * equals fg_spmm_csr_general_f32.  One launch per column block of the plan,
+ * the partial fold carried in `out`.
+ */
+FG_API int fg_spmm_csr_mh_general_f32(const fg_spmm_plan *plan, const float *feat, const float *w, float *out,
+                                      int32_t H, int32_t D, int32_t msg, int32_t reduce, void *stream);
+
+/*
  * Out[e] = sum_k src[col[e], k] * dst[row[e], k]   (op/vanilla_sddmm.py:43-47;
  * note src is indexed by COLUMN ids and dst by ROW ids, as the reference's
  * tests shape them: tests/test_module_sddmm.py:18-19).
@@ -252,10 +267,32 @@ FG_API int fg_sddmm_coo_general_plan_f32(const fg_sddmm_plan *plan, const float 
  * The edge list is the CSR one: row r's edges are [indptr[r], indptr[r+1]).
  * out[e, h] = exp(scores[e, h] - max) / sum over the row's edges of
  * exp(scores[e', h] - max), max taken over the same edges, per head.  scores
- * and out are [nnz, H] and may be the same buffer.  Scores must be finite.
+ * and out are [nnz, H] and may be the same buffer.  A score of -inf is a masked
+ * edge: weight 0 wherever it stands in the row; a row and head with nothing
+ * but -inf gives NaN (0 / 0), as the textbook softmax does.
  */
 FG_API int fg_edge_softmax_csr_f32(int64_t n_rows, const int32_t *indptr, const float *scores, float *out, int32_t H,
                                    void *stream);
+/*
+ * Backward of the edge softmax (no counterpart in the reference): with
+ * `weights` the output of fg_edge_softmax_csr_f32 and `grad` the gradient that
+ * arrives for it, both [nnz, H],
+ *   out[e, h] = weights[e, h] * (grad[e, h] - sum over the row's edges e' of weights[e', h] * grad[e', h]),
+ * the gradient for the scores.  out may be the same buffer as grad.
+ */
+FG_API int fg_edge_softmax_backward_csr_f32(int64_t n_rows, const int32_t *indptr, const float *weights,
+                                            const float *grad, float *out, int32_t H, void *stream);
+/*
+ * Helpers of the multi-head backward (no counterpart in the reference).
+ * fg_permute_rows_f32: out[i, :] = in[perm[i], :] for i in [0, n), rows of
+ * `width` floats; carries per-edge weights from the order of a matrix's CSR
+ * arrays to that of its transpose's.  perm entries must lie in [0, rows of
+ * in); in and out must not overlap.  fg_add_f32: out[i] = a[i] + b[i] for
+ * i in [0, n); out may be a or b.
+ */
+FG_API int fg_permute_rows_f32(int64_t n, int32_t width, const int32_t *perm, const float *in, float *out,
+                               void *stream);
+FG_API int fg_add_f32(int64_t n, const float *a, const float *b, float *out, void *stream);
 /*
  * fg_sddmm_coo_mh_f32 followed by fg_edge_softmax_csr_f32, on the plan's edge
  * list, which must be row-sorted (FG_EUNSUPPORTED otherwise):

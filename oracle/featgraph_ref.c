@@ -359,3 +359,66 @@ int fgref_edge_softmax(int64_t n_dst, int64_t H, const int32_t *indptr, const fl
   }
   return FGREF_OK;
 }
+
+/* Multi-head generalised SpMM (not in the reference): fgref_spmm_general with a
+ * per-edge per-head weight, the message slot of op/vanilla_spmm.py:46-53 applied
+ * head by head on [N,H,D] features:
+ *   term(e, h, d) = msg(Src[indices[e], h, d], W[e, h]),  Out[r, h, d] = fold over e in CSR order.
+ * Same folds as fgref_spmm_general (first term assigned for max / min, mean = sum / degree,
+ * rows without nonzeros 0).  (mul, sum) is fgref_spmm_mh bit for bit; H = 1 is fgref_spmm_general. */
+int fgref_spmm_mh_general(int64_t n_dst, int64_t H, int64_t D, const int32_t *indptr, const int32_t *indices,
+                          const float *w, const float *src, float *out, int msg, int reduce) {
+  if (n_dst < 0 || H <= 0 || D <= 0 || msg < 0 || msg > 4 || reduce < 0 || reduce > 3) return FGREF_EINVAL;
+  const int64_t F = H * D;
+#pragma omp parallel for schedule(dynamic, 64)
+  for (int64_t r = 0; r < n_dst; ++r) {
+    float *acc = out + r * F;
+    const int64_t lo = indptr[r], hi = indptr[r + 1];
+    for (int64_t f = 0; f < F; ++f) acc[f] = 0.0f;
+    for (int64_t e = lo; e < hi; ++e) {
+      const float *x = src + (int64_t)indices[e] * F;
+      for (int64_t h = 0; h < H; ++h) {
+        const float v = msg == 4 ? 0.0f : w[e * H + h];
+        for (int64_t d = 0; d < D; ++d) {
+          const int64_t f = h * D + d;
+          const float t = fgref_msg(msg, x[f], v);
+          if (reduce == 0 || reduce == 3)
+            acc[f] = acc[f] + t;
+          else if (e == lo)
+            acc[f] = t;
+          else if (reduce == 1)
+            acc[f] = (t > acc[f]) ? t : acc[f];
+          else
+            acc[f] = (t < acc[f]) ? t : acc[f];
+        }
+      }
+    }
+    if (reduce == 3 && hi > lo) {
+      const float n = (float)(hi - lo);
+      for (int64_t f = 0; f < F; ++f) acc[f] = acc[f] / n;
+    }
+  }
+  return FGREF_OK;
+}
+
+/* Backward of the edge softmax (not in the reference; the step between the
+ * gradients of multi-head SpMM and multi-head SDDMM in a GAT layer).  With
+ * A = softmax of the scores over a destination row's edges (per head) and G the
+ * gradient that arrives for A, the gradient for the scores is
+ *   dS[e, h] = A[e, h] * (G[e, h] - sum_{e' in the row} A[e', h] * G[e', h]).
+ * Computed in binary64 from the float32 inputs and rounded once. */
+int fgref_edge_softmax_backward(int64_t n_dst, int64_t H, const int32_t *indptr, const float *weights,
+                                const float *grad, float *out) {
+  if (n_dst < 0 || H <= 0) return FGREF_EINVAL;
+#pragma omp parallel for schedule(dynamic, 64)
+  for (int64_t r = 0; r < n_dst; ++r) {
+    const int64_t lo = indptr[r], hi = indptr[r + 1];
+    for (int64_t h = 0; h < H; ++h) {
+      double dot = 0.0;
+      for (int64_t e = lo; e < hi; ++e) dot += (double)weights[e * H + h] * (double)grad[e * H + h];
+      for (int64_t e = lo; e < hi; ++e)
+        out[e * H + h] = (float)((double)weights[e * H + h] * ((double)grad[e * H + h] - dot));
+    }
+  }
+  return FGREF_OK;
+}

@@ -33,7 +33,7 @@ def lib():
         _lib = ctypes.CDLL(_LIB_PATH)
         for name in ("fgref_spmm_csr_x86", "fgref_spmm_dds_x86", "fgref_sddmm_x86", "fgref_sddmm_x86_fast",
                      "fgref_spmm_csr_f64", "fgref_sddmm_f64", "fgref_sddmm_mh", "fgref_spmm_mh", "fgref_spmm_general",
-                     "fgref_sddmm_general", "fgref_edge_softmax"):
+                     "fgref_sddmm_general", "fgref_edge_softmax", "fgref_spmm_mh_general", "fgref_edge_softmax_backward"):
             getattr(_lib, name).restype = ctypes.c_int
     return _lib
 
@@ -192,6 +192,62 @@ def edge_softmax(indptr, scores):
     _check(lib().fgref_edge_softmax(_i64(n_dst), _i64(H), _ptr(indptr), _ptr(scores), _ptr(out)),
            "fgref_edge_softmax")
     return out
+
+
+def spmm_mh_general(indptr, indices, w, src, msg="mul", reduce="sum"):
+    """Multi-head generalised SpMM: w [nnz,H], src [N,H,D] -> fold of msg(src[col,h,:], w[e,h]) per row and head."""
+    indptr, indices = _arr(indptr, np.int32), _arr(indices, np.int32)
+    w, src = _arr(w, np.float32), _arr(src, np.float32)
+    n_dst, (_, H, D) = indptr.shape[0] - 1, src.shape
+    assert w.shape == (indices.shape[0], H)
+    out = np.empty((n_dst, H, D), dtype=np.float32)
+    _check(lib().fgref_spmm_mh_general(_i64(n_dst), _i64(H), _i64(D), _ptr(indptr), _ptr(indices), _ptr(w),
+                                       _ptr(src), _ptr(out), ctypes.c_int(MSG_OPS[msg]),
+                                       ctypes.c_int(REDUCE_OPS[reduce])), "fgref_spmm_mh_general")
+    return out
+
+
+def edge_softmax_backward(indptr, weights, grad):
+    """Gradient for the scores of an edge softmax: weights * (grad - rowsum(weights * grad)), binary64 inside."""
+    indptr, weights, grad = _arr(indptr, np.int32), _arr(weights, np.float32), _arr(grad, np.float32)
+    assert weights.shape == grad.shape
+    n_dst, H = indptr.shape[0] - 1, weights.shape[1]
+    out = np.empty_like(weights)
+    _check(lib().fgref_edge_softmax_backward(_i64(n_dst), _i64(H), _ptr(indptr), _ptr(weights), _ptr(grad),
+                                             _ptr(out)), "fgref_edge_softmax_backward")
+    return out
+
+
+def attention_mh_backward(indptr, indices, key, query, value, dout):
+    """Gradients (d_key, d_query, d_value) of attention_mh, composed from the checkers above.
+
+    With A the attention weights, row[e] the destination row of edge e and T the transposed matrix:
+      d_value[c] = sum_{e: col=c} A[e] * dout[row[e]]      spmm_mh over T with the weights in T's order
+      G[e]       = <dout[row[e]], value[col[e]]>           sddmm_mh
+      dS         = edge_softmax_backward(A, G)
+      d_query[r] = sum_{e in row r} dS[e] * key[col[e]]    spmm_mh
+      d_key[c]   = sum_{e: col=c} dS[e] * query[row[e]]    spmm_mh over T
+    value None means key is also the value matrix: then d_key carries both contributions.
+    """
+    import scipy.sparse
+    indptr, indices = _arr(indptr, np.int32), _arr(indices, np.int32)
+    n_dst, n_src, nnz = indptr.shape[0] - 1, key.shape[0], indices.shape[0]
+    row = np.repeat(np.arange(n_dst, dtype=np.int32), np.diff(indptr))
+    weights = edge_softmax(indptr, sddmm_mh(row, indices, key, query))
+    # transposed structure; `perm` lists the edges in the transposed matrix's CSR order (stable: by column, then CSR order)
+    perm = np.argsort(indices, kind="stable")
+    t_indptr = np.zeros(n_src + 1, dtype=np.int32)
+    np.cumsum(np.bincount(indices, minlength=n_src), out=t_indptr[1:])
+    t_indices = row[perm]
+    val = key if value is None else value
+    d_value = spmm_mh(t_indptr, t_indices, np.ascontiguousarray(weights[perm]), dout)
+    grad_w = sddmm_mh(row, indices, val, dout)
+    d_scores = edge_softmax_backward(indptr, weights, grad_w)
+    d_query = spmm_mh(indptr, indices, d_scores, key)
+    d_key = spmm_mh(t_indptr, t_indices, np.ascontiguousarray(d_scores[perm]), query)
+    if value is None:
+        return d_key + d_value, d_query, None
+    return d_key, d_query, d_value
 
 
 def attention_mh(indptr, indices, key, query, value=None):

@@ -400,3 +400,105 @@ def test_attention_against_dense_masked_softmax():
         got = ref.attention_mh(adj.indptr, adj.indices, key, query, val)
         np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
     assert (np.diff(adj.indptr) == 0).any() and not got[np.diff(adj.indptr) == 0].any()
+
+
+# ---------------------------------------------------------------- multi-head generalised SpMM, softmax backward
+@pytest.mark.parametrize("msg", ["mul", "add", "sub", "div", "copy_u"])
+@pytest.mark.parametrize("reduce", ["sum", "max", "min", "mean"])
+def test_multi_head_generalised_spmm_against_numpy_reduceat_per_head(msg, reduce):
+    """Per head np.add / maximum / minimum.reduceat over exact terms (small integers, weights 1, 2, 4)."""
+    adj, _ = _int_case(seed=6)
+    H, D = 3, 5
+    rng = np.random.default_rng(8)
+    feat = rng.integers(-4, 5, (adj.shape[1], H, D)).astype(np.float32)
+    w = rng.choice(np.array([1, 2, 4], np.float32), (adj.nnz, H))
+    out = ref.spmm_mh_general(adj.indptr, adj.indices, w, feat, msg, reduce)
+    rows = _rows_with_edges(adj)
+    for h in range(H):
+        u, e = feat[adj.indices, h].astype(np.float64), w[:, h].astype(np.float64)[:, None]
+        terms = {"mul": u * e, "add": u + e, "sub": u - e, "div": u / e, "copy_u": u}[msg]
+        fold = {"sum": np.add, "mean": np.add, "max": np.maximum, "min": np.minimum}[reduce].reduceat(
+            terms, adj.indptr[rows], axis=0)
+        if reduce == "mean":
+            fold = fold / np.diff(adj.indptr)[rows][:, None]
+            np.testing.assert_allclose(out[rows, h], fold, rtol=1e-6, atol=0)
+        else:
+            assert np.array_equal(out[rows, h], fold.astype(np.float32))
+    assert np.all(out[np.diff(adj.indptr) == 0] == 0)
+
+
+def test_multi_head_generalised_spmm_reduces_to_its_relatives(adj_127x255):
+    adj = adj_127x255
+    rng = np.random.default_rng(9)
+    feat = rng.standard_normal((adj.shape[1], 4, 6), dtype=np.float32)
+    w = rng.random((adj.nnz, 4), dtype=np.float32) + np.float32(0.5)
+    # (mul, sum) is the multi-head operator of config 5 bit for bit
+    assert np.array_equal(ref.spmm_mh_general(adj.indptr, adj.indices, w, feat, "mul", "sum"),
+                          ref.spmm_mh(adj.indptr, adj.indices, w, feat))
+    # one head is the single-head generalised operator
+    for msg, reduce in (("add", "max"), ("div", "mean"), ("sub", "min")):
+        one = ref.spmm_mh_general(adj.indptr, adj.indices, w[:, :1].copy(), feat[:, :1].copy(), msg, reduce)
+        assert np.array_equal(one[:, 0], ref.spmm_general(adj.indptr, adj.indices, w[:, 0].copy(),
+                                                          feat[:, 0].copy(), msg, reduce))
+    # heads never mix: head 2 of the 4-head result equals the operator run on head 2 alone
+    full = ref.spmm_mh_general(adj.indptr, adj.indices, w, feat, "mul", "max")
+    alone = ref.spmm_general(adj.indptr, adj.indices, w[:, 2].copy(), feat[:, 2].copy(), "mul", "max")
+    assert np.array_equal(full[:, 2], alone)
+
+
+def test_edge_softmax_backward_against_torch_autograd_and_identities():
+    """The gradient formula against a library routine (torch.softmax's own backward, float64, per row) and what the
+    mathematics fixes: the gradients of a row sum to zero (the weights sum to one whatever the scores), and a
+    gradient that is constant over a row gives zero."""
+    import torch
+    adj = datasets.config_graph("c4-mini")
+    H = 3
+    rng = np.random.default_rng(12)
+    scores = (rng.standard_normal((adj.nnz, H)) * 2).astype(np.float32)
+    grad = rng.standard_normal((adj.nnz, H)).astype(np.float32)
+    weights = ref.edge_softmax(adj.indptr, scores)
+    got = ref.edge_softmax_backward(adj.indptr, weights, grad)
+    for r in (0, 3, 29, 1000, adj.shape[0] - 1):
+        sl = slice(adj.indptr[r], adj.indptr[r + 1])
+        s = torch.tensor(scores[sl], dtype=torch.float64, requires_grad=True)
+        torch.softmax(s, dim=0).backward(torch.tensor(grad[sl], dtype=torch.float64))
+        np.testing.assert_allclose(got[sl], s.grad.numpy(), rtol=2e-5, atol=1e-7)
+    rows = _rows_with_edges(adj)
+    sums = np.add.reduceat(got.astype(np.float64), adj.indptr[rows], axis=0)
+    np.testing.assert_allclose(sums, 0.0, atol=1e-6)
+    const = np.repeat(rng.standard_normal((adj.shape[0], H)).astype(np.float32), np.diff(adj.indptr), axis=0)
+    np.testing.assert_allclose(ref.edge_softmax_backward(adj.indptr, weights, const), 0.0, atol=1e-6)
+    # a wrong sign or a dropped row term would survive neither check; a single-edge row has gradient exactly 0
+    single = np.flatnonzero(np.diff(adj.indptr) == 1)
+    assert single.size and np.all(got[adj.indptr[single]] == 0)
+
+
+@pytest.mark.parametrize("shared", [False, True])
+def test_attention_backward_against_torch_autograd_of_the_dense_form(shared):
+    """All three gradients of the composed attention checker against torch's autograd of the textbook dense form
+    softmax(mask(Q K^T)) V in float64 (a matrix small enough to densify; rows without entries included)."""
+    import torch
+    rng = np.random.default_rng(13)
+    adj = scipy.sparse.random(23, 31, density=0.2, format="lil", random_state=rng)
+    adj[4] = 0
+    adj = adj.tocsr()
+    adj.sort_indices()
+    H, D = 2, 4
+    key = rng.standard_normal((31, H, D), dtype=np.float32)
+    value = None if shared else rng.standard_normal((31, H, D), dtype=np.float32)
+    query = rng.standard_normal((23, H, D), dtype=np.float32)
+    dout = rng.standard_normal((23, H, D), dtype=np.float32)
+    d_key, d_query, d_value = ref.attention_mh_backward(adj.indptr, adj.indices, key, query, value, dout)
+    k = torch.tensor(key, dtype=torch.float64, requires_grad=True)
+    q = torch.tensor(query, dtype=torch.float64, requires_grad=True)
+    v = k if shared else torch.tensor(value, dtype=torch.float64, requires_grad=True)
+    mask = torch.tensor(adj.toarray() != 0)
+    s = torch.einsum("rhd,chd->hrc", q, k).masked_fill(~mask[None], float("-inf"))
+    a = torch.nan_to_num(torch.softmax(s, dim=2))                       # rows without entries: all zero
+    out = torch.einsum("hrc,chd->rhd", a, v)
+    out.backward(torch.tensor(dout, dtype=torch.float64))
+    np.testing.assert_allclose(d_key, k.grad.numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(d_query, q.grad.numpy(), rtol=1e-4, atol=1e-5)
+    if not shared:
+        np.testing.assert_allclose(d_value, v.grad.numpy(), rtol=1e-4, atol=1e-5)
+    assert not d_query[4].any()
