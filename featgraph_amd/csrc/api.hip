@@ -303,7 +303,7 @@ int multi_run(const fg_spmm_plan *plan, const fg::MultiRuns *runs, fg::SpmmArgs 
   const int64_t n = plan->n_rows;
   auto long_split = [&](int pass) {
     a.long_runs = runs->long_runs[pass];
-    a.long_blocks = std::min((a.long_runs + fg::kWavesPerBlock - 1) / fg::kWavesPerBlock, 2048);
+    a.long_blocks = std::min(a.long_runs, 2048);  // one workgroup per long run at a time
   };
   if (runs->passes == 1) {
     a.runs = runs->rec;

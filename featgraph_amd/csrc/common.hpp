@@ -66,7 +66,7 @@ struct SpmmArgs {
   int32_t accumulate = 0;
   // several-rows-per-wave kernel: one pass's records {first nonzero, one past the last, row id, 0}, n_rows of them
   const int4 *runs = nullptr;
-  int32_t long_runs = 0;    // the first long_runs records are long runs: one wave each, in the first
+  int32_t long_runs = 0;    // the first long_runs records are long runs: one workgroup each, in the first
   int32_t long_blocks = 0;  // long_blocks workgroups of the grid
   int32_t interleave_tiles = 1;  // this many tiles alternate workgroup by workgroup along grid.x; the rest along grid.y
   // records over a re-laid copy of the ids (MultiRuns::ids_p): `indices` is that copy, and a run's values start

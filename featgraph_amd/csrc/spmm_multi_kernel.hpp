@@ -25,7 +25,7 @@
 // carried sums of item k+1, record of item k+2; within an item the next batch
 // of ids is asked for behind the current batch's first gathers (loads return in
 // order, so the adds wait only for the gathers).  Runs of kLongRun nonzeros or
-// more take the one-wave-per-run path below instead.
+// more take the one-workgroup-per-run path below instead.
 //
 // RED / MSG turn the multiply-add into the generalised operator (README.md:6 of the reference): term =
 // MSG(feature, value), folded with RED in the same order; a picking reducer (max / min) takes a row's first
@@ -44,8 +44,10 @@
 namespace fg {
 namespace {
 
-// Runs of at least this many nonzeros go to the one-wave-per-run path (spmm.multi_long overrides).
-constexpr uint32_t kLongRun = 512;
+// Runs of at least this many nonzeros go to the one-workgroup-per-run path (spmm.multi_long overrides).  Measured on
+// the 232,965-vertex graph at 16 / 32 / 64 floats: 512: 1.19 / 1.08 / 1.80 ms, 1024: 1.00 / 0.99 / 1.78, 2048: 1.14 / 1.33 / 2.10
+// (below it the workgroups idle at their barriers too often, above it the chains of the several-rows path set the time).
+constexpr uint32_t kLongRun = 1024;
 
 template <int... Js, typename F>
 __device__ __forceinline__ void static_for(std::integer_sequence<int, Js...>, F f) {
@@ -159,124 +161,125 @@ struct alignas(4) Float4U {
 // Long runs.  A row's sum is a chain: its nonzeros are added one after the other, so a kernel that keeps k
 // gathers of a row in flight cannot finish a run of L nonzeros sooner than L / k memory round trips, and on a
 // power-law graph the longest rows then set the time of the whole launch (most visibly at short feature
-// lengths, where everything else is quick).  Here one wave works on ONE run: its 64/G groups take 64/G
-// consecutive nonzeros per round, so the gathers and the (rounded) products of many nonzeros proceed at once,
-// and only the adds stay ordered: the products go through LDS to the first 4*G lanes, lane i of which owns
-// float i of the tile and adds its terms one by one.  Same terms, same order, same roundings as everywhere else.
-constexpr int kLongRounds = 8;  // rounds per batch of the long-run path; two batches alternate
+// lengths, where everything else is quick: on the 232,965-vertex benchmark graph at 32 floats the rows beyond
+// 8,192 nonzeros, 0.2 % of the matrix, cost a sixth of the time while one wave worked on each of their runs).
+// Here a whole WORKGROUP works on ONE run.  Per step each of its four waves takes the next kLongRounds * 64/G
+// consecutive nonzeros: its 64/G groups gather 64/G of them per round, so the gathers and the (rounded) products
+// of four waves x kLongRounds rounds proceed at once, and only the adds stay ordered: the products go through LDS
+// to the first 4*G lanes of the first wave, lane i of which owns float i of the tile and adds its terms one by
+// one, the waves' regions in turn.  Same terms, same order, same roundings as everywhere else.
+constexpr int kLongRounds = 8;  // rounds per wave and step; the gathers of two steps are in flight per wave
 
 template <int G, bool BUF, bool U24, int RED, int MSG>
-__device__ __forceinline__ void spmm_long_runs(const SpmmArgs &a, const FeatRows<BUF, U24> &feat, int wave, int n_waves,
-                                               int lane, uint32_t lane_bytes, float *lds, int tile) {
+__device__ __forceinline__ void spmm_long_runs(const SpmmArgs &a, const FeatRows<BUF, U24> &feat, int first_run,
+                                               int run_stride, int lane, int wave, uint32_t lane_bytes, float *lds,
+                                               int tile) {
   constexpr int NG = kWaveSize / G;   // nonzeros per round
   constexpr int TW = 4 * G;           // floats per tile
   constexpr int R = kLongRounds;
-  constexpr int BLK = 256;            // nonzeros per block of ids: lane l holds ids l, 64 + l, 128 + l, 192 + l
-  constexpr int NB = BLK / NG / R;    // batches per block
+  constexpr int RB = R * NG;          // nonzeros per wave and step
+  constexpr int SB = kWavesPerBlock * RB;       // nonzeros per step
+  constexpr int Q = (RB + kWaveSize - 1) / kWaveSize;  // ids per lane and step: lane l holds ids l, 64 + l, ...
+  constexpr int REGION = R * 256;     // floats of LDS per wave: R rounds x 64 lanes x float4
+  constexpr bool HAS_VALS = RED < 0 || MSG != FG_MSG_COPY_U;
   const int g = lane / G;
   const int64_t F = a.F;
   const bool carry = a.accumulate != 0;
   const int f1 = (a.tile_base + tile) * TW + lane;  // the float this lane sums
-  const bool owner = lane < TW && f1 < a.F;
-
-  int vo = 0;  // from a nonzero's place in the id array to its place in the value array
-  auto load_ids = [&](int e, int rem, Ids &d) {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      d.c[q] = 0;
-      d.v[q] = 0.0f;
-      if (64 * q + lane < rem) {
-        d.c[q] = a.indices[e + 64 * q + lane];
-        if (RED < 0 || MSG != FG_MSG_COPY_U) d.v[q] = a.w[e + vo + 64 * q + lane];
-      }
-    }
-  };
-  // round t of a block covers its nonzeros NG*t .. NG*t + NG - 1, one per group
-  auto issue = [&](float4(&x)[R], auto b, const Ids &d, int cnt) {
-    static_for(std::make_integer_sequence<int, R>{}, [&](auto r) {
-      constexpr int t = decltype(b)::value * R + decltype(r)::value;
-      constexpr int q = NG * t / 64, l0 = NG * t % 64;
-      if (decltype(r)::value == 0 || NG * t < cnt) {
-        const int c = __builtin_amdgcn_ds_bpermute((l0 + g) << 2, d.c[q]);  // past the run's end: id 0, never added
-        x[r] = feat.load(c, lane_bytes);
-      }
-    });
-  };
-  // assign: the block starts the row and the reducer picks, so the very first term is taken as it is
-  auto consume = [&](const float4(&x)[R], auto b, const Ids &d, int cnt, float &acc, bool assign) {
-    static_for(std::make_integer_sequence<int, R>{}, [&](auto r) {
-      constexpr int t = decltype(b)::value * R + decltype(r)::value;
-      constexpr int q = NG * t / 64, l0 = NG * t % 64;
-      if (NG * t < cnt) {
-        const float v = __int_as_float(__builtin_amdgcn_ds_bpermute((l0 + g) << 2, __float_as_int(d.v[q])));
-        // lane (g, gl) holds floats 4*gl .. 4*gl+3 of nonzero g: float index g*TW + 4*gl = 4*lane
-        if constexpr (RED < 0)
-          *reinterpret_cast<float4 *>(lds + decltype(r)::value * 256 + 4 * lane) =
-              make_float4(v * x[r].x, v * x[r].y, v * x[r].z, v * x[r].w);
-        else
-          *reinterpret_cast<float4 *>(lds + decltype(r)::value * 256 + 4 * lane) =
-              make_float4(message_of<MSG>(x[r].x, v), message_of<MSG>(x[r].y, v), message_of<MSG>(x[r].z, v),
-                          message_of<MSG>(x[r].w, v));
-      }
-    });
-    // The products were stored with one lane mapping and are read back with another.  LDS serves a wave's
-    // accesses in order; the fence and the barrier keep the compiler from moving the reads above the stores.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    if (lane < TW) {
-      static_for(std::make_integer_sequence<int, R>{}, [&](auto r) {
-        constexpr int t = decltype(b)::value * R + decltype(r)::value;
-#pragma unroll
-        for (int h = 0; h < NG; ++h)
-          if (NG * t + h < cnt) {  // wave-uniform test
-            const float term = lds[decltype(r)::value * 256 + h * TW + lane];
-            if constexpr (RED < 0)
-              acc = acc + term;
-            else if ((RED == FG_REDUCE_MAX || RED == FG_REDUCE_MIN) && t == 0 && h == 0)
-              acc = assign ? term : fold_of<RED>(acc, term);
-            else
-              acc = fold_of<RED>(acc, term);
-          }
-      });
-    }
-    // ... and the next batch's stores below these reads
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+  const bool adder = wave == 0 && lane < TW && f1 < a.F;
+  float *const mine = lds + wave * REGION;
+  struct StepIds {
+    int c[Q];
+    float v[Q];
   };
 
-  for (int it = wave; it < a.long_runs; it += n_waves) {
+  for (int it = first_run; it < a.long_runs; it += run_stride) {  // the same for all four waves
     const int4 rec = a.runs[it];
-    const int lo = rec.x, hi = rec.y, row = rec.z;
-    if (hi <= lo) continue;
-    vo = a.vals_by_csr ? rec.w - rec.x : 0;
+    const int lo = rec.x, len = rec.y - rec.x, row = rec.z;
+    if (len <= 0) continue;
+    const int vo = a.vals_by_csr ? rec.w - rec.x : 0;  // from a nonzero's place in the id array to its value's
     // a picking reducer takes the row's first term as it is instead of comparing it with a carried value
     bool starts = false;
     if constexpr (RED == FG_REDUCE_MAX || RED == FG_REDUCE_MIN) starts = (a.vals_by_csr ? rec.w : rec.x) == a.indptr[row];
     float acc = 0.0f;
-    float4 xa[R], xb[R];
-    Ids ids_a;
-    load_ids(lo, hi - lo, ids_a);
-    if (carry && owner && !starts) acc = a.out[static_cast<int64_t>(row) * F + f1];
-    issue(xa, std::integral_constant<int, 0>{}, ids_a, min(BLK, hi - lo));
-    for (int e = lo; e < hi; e += BLK) {
-      const int cnt = min(BLK, hi - e);
-      const bool more = hi - e > BLK;
-      Ids ids_n;
-      load_ids(e + BLK, hi - e - BLK, ids_n);  // the next block's ids, behind this block's first gathers
-      static_for(std::make_integer_sequence<int, NB>{}, [&](auto b) {
-        constexpr int bi = decltype(b)::value;
-        float4(&xc)[R] = (bi & 1) ? xb : xa;
-        float4(&xn)[R] = (bi & 1) ? xa : xb;
-        if constexpr (bi + 1 < NB) {
-          if (NG * R * (bi + 1) < cnt) issue(xn, std::integral_constant<int, bi + 1>{}, ids_a, cnt);
-        } else {
-          if (more) issue(xn, std::integral_constant<int, 0>{}, ids_n, hi - e - BLK);  // NB is even: xn is xa again
+    if (carry && adder && !starts) acc = a.out[static_cast<int64_t>(row) * F + f1];
+
+    // this wave's nonzeros of step s: RB of them from `at(s)` on, as many as the run still has
+    auto at = [&](int s) { return s * SB + wave * RB; };
+    auto load_ids = [&](int s, StepIds &d) {
+      const int e = lo + at(s), rem = len - at(s);
+#pragma unroll
+      for (int q = 0; q < Q; ++q) {
+        d.c[q] = 0;  // past the run's end: id 0, a valid row to gather from, never added
+        d.v[q] = 0.0f;
+        if (kWaveSize * q + lane < min(rem, RB)) {
+          d.c[q] = a.indices[e + kWaveSize * q + lane];
+          if (HAS_VALS) d.v[q] = a.w[e + vo + kWaveSize * q + lane];
         }
-        if (NG * R * bi < cnt) consume(xc, b, ids_a, cnt, acc, bi == 0 && starts && e == lo);
+      }
+    };
+    // round r of a step covers the wave's nonzeros NG*r .. NG*r + NG - 1, one per group
+    auto issue = [&](float4(&x)[R], const StepIds &d, int cnt) {
+      static_for(std::make_integer_sequence<int, R>{}, [&](auto r) {
+        constexpr int j0 = NG * decltype(r)::value, q = j0 / kWaveSize, l0 = j0 % kWaveSize;
+        if (j0 < cnt) x[r] = feat.load(__builtin_amdgcn_ds_bpermute((l0 + g) << 2, d.c[q]), lane_bytes);
       });
-      ids_a = ids_n;
+    };
+    auto products = [&](const float4(&x)[R], const StepIds &d, int cnt) {
+      static_for(std::make_integer_sequence<int, R>{}, [&](auto r) {
+        constexpr int j0 = NG * decltype(r)::value, q = j0 / kWaveSize, l0 = j0 % kWaveSize;
+        if (j0 < cnt) {
+          const float v = __int_as_float(__builtin_amdgcn_ds_bpermute((l0 + g) << 2, __float_as_int(d.v[q])));
+          // lane (g, gl) holds floats 4*gl .. 4*gl+3 of nonzero g: float index g*TW + 4*gl = 4*lane
+          float4 t;
+          if constexpr (RED < 0)
+            t = make_float4(v * x[r].x, v * x[r].y, v * x[r].z, v * x[r].w);
+          else
+            t = make_float4(message_of<MSG>(x[r].x, v), message_of<MSG>(x[r].y, v), message_of<MSG>(x[r].z, v),
+                            message_of<MSG>(x[r].w, v));
+          *reinterpret_cast<float4 *>(mine + decltype(r)::value * 256 + 4 * lane) = t;
+        }
+      });
+    };
+    auto count = [&](int s) { return max(0, min(RB, len - at(s))); };
+
+    const int n_steps = (len + SB - 1) / SB;
+    float4 xa[R], xb[R];
+    StepIds ids_cur, ids_nxt;
+    load_ids(0, ids_cur);
+    issue(xa, ids_cur, count(0));
+    load_ids(1, ids_nxt);
+    // One step: the next step's gathers go out first, then this step's products go to LDS, the first wave adds
+    // them in order, and the regions are free again.  Every wave passes both barriers of every step.
+    auto step = [&](int s, float4(&cur)[R], float4(&nxt)[R]) {
+      issue(nxt, ids_nxt, count(s + 1));
+      StepIds ids_after;
+      load_ids(s + 2, ids_after);
+      products(cur, ids_cur, count(s));
+      __syncthreads();
+      if (wave == 0 && lane < TW) {
+        const int here = min(SB, len - s * SB);
+#pragma unroll 8
+        for (int t = 0; t < here; ++t) {
+          const int w = t / RB, j = t % RB;
+          const float term = lds[w * REGION + (j / NG) * 256 + (j % NG) * TW + lane];
+          if constexpr (RED < 0)
+            acc = acc + term;
+          else if ((RED == FG_REDUCE_MAX || RED == FG_REDUCE_MIN) && starts && s == 0 && t == 0)
+            acc = term;
+          else
+            acc = fold_of<RED>(acc, term);
+        }
+      }
+      __syncthreads();
+      ids_cur = ids_nxt;
+      ids_nxt = ids_after;
+    };
+    for (int s = 0; s < n_steps; s += 2) {
+      step(s, xa, xb);
+      if (s + 1 < n_steps) step(s + 1, xb, xa);
     }
-    if (owner) a.out[static_cast<int64_t>(row) * F + f1] = acc;
+    if (adder) a.out[static_cast<int64_t>(row) * F + f1] = acc;
   }
 }
 
@@ -303,11 +306,11 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(3
   const uint32_t lane_bytes = static_cast<uint32_t>(fok ? f0 : a.F - 4) * 4u;
   const FeatRows<BUF, U24> feat(a.feat, a.n_cols, F);
   const bool carry = a.accumulate != 0;
-  // the first workgroups take the long runs (the records come by descending length), one wave per run
+  // the first workgroups take the long runs (the records come by descending length), one workgroup per run
   if (bx < a.long_blocks) {
-    __shared__ float products[kWavesPerBlock][kLongRounds * 256];  // per wave: a batch of rounds x 64 lanes x float4
-    spmm_long_runs<G, BUF, U24, RED, MSG>(a, feat, static_cast<int>(bx * kWavesPerBlock + (threadIdx.x >> 6)),
-                      a.long_blocks * kWavesPerBlock, lane, lane_bytes, products[threadIdx.x >> 6], tile);
+    __shared__ float products[kWavesPerBlock * kLongRounds * 256];  // per wave: rounds x 64 lanes x float4
+    spmm_long_runs<G, BUF, U24, RED, MSG>(a, feat, bx, a.long_blocks, lane, static_cast<int>(threadIdx.x >> 6),
+                                          lane_bytes, products, tile);
     return;
   }
   const int n_waves = (gx - a.long_blocks) * kWavesPerBlock;

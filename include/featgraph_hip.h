@@ -423,8 +423,8 @@ FG_API int64_t fg_probe_store_rows_f32(float *out, int64_t n_out_rows, int32_t r
  * "spmm.multi" (0/1: never / always use the several-rows-per-wave kernel where
  * it applies; by default it runs unless one of the shape keys above is set;
  * read at plan creation and at launch), "spmm.multi_blocks" (its grid size),
- * "spmm.multi_long" (run length from which a run gets a wave of its own,
- * default 512; read at plan creation), "spmm.tile_interleave" (feature tiles
+ * "spmm.multi_long" (run length from which a run gets a workgroup of its
+ * own, default 1024; read at plan creation), "spmm.tile_interleave" (feature tiles
  * whose workgroups alternate inside one launch of that kernel: 1 or 2, default 2),
  * "spmm.general_multi" (0/1: whether fg_spmm_csr_general_f32 may use that
  * kernel; default 1), "spmm.relay" (0/1: whether the plan keeps, per pass layout of that kernel, a

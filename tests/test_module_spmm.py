@@ -285,7 +285,7 @@ def test_rows_per_wave_kernel_gives_the_same_bits(config_guard, blocks, long_run
     adj = datasets.config_graph("c2-mini")
     _lib.config_set("spmm.blocked", blocks[0])
     _lib.config_set("spmm.block_cols", blocks[1])
-    _lib.config_set("spmm.multi_long", long_run)       # 8: nearly every run takes the one-wave-per-run path; 2^20: none
+    _lib.config_set("spmm.multi_long", long_run)       # 8: nearly every run takes the one-workgroup-per-run path; 2^20: none
     module = VanillaSpMMhip(adj)
     for F in (4, 8, 16, 20, 32, 36, 64, 68, 200, 512):
         feat = datasets.spmm_operands(adj, F)
