@@ -189,7 +189,11 @@ int multi_runs_build(const int32_t *seg, const int32_t *row_order, const int32_t
 }
 
 bool spmm_multi_applies(const SpmmArgs &a) {
-  return a.H == 1 && a.F % 4 == 0 && a.F >= 4 && aligned_to(a.feat, 16) && aligned_to(a.out, 16);
+  // Any feature length from four floats on whose last tile holds none or at least four floats (a lane that the
+  // row's end cuts takes the row's last four floats, which must lie in its own tile); rows that are not 16-byte
+  // aligned are read with 4-byte aligned accesses.
+  const int rest = a.F % spmm_multi_tile(a.F);
+  return a.H == 1 && a.F >= 4 && (rest == 0 || rest >= 4) && aligned_to(a.feat, 4) && aligned_to(a.out, 4);
 }
 
 bool spmm_multi_general_applies(const SpmmArgs &a) {

@@ -74,6 +74,19 @@ __device__ __forceinline__ int group_bcast(int x, bool hi_half) {
   }
 }
 
+// Four adjacent floats at an address that is only known to be 4-byte aligned (feature rows whose length is not a
+// multiple of four floats start anywhere): one 16-byte access where the address allows it.
+struct alignas(4) Float4A {
+  float x, y, z, w;
+};
+__device__ __forceinline__ float4 load4(const float *p) {
+  const Float4A q = *reinterpret_cast<const Float4A *>(p);
+  return make_float4(q.x, q.y, q.z, q.w);
+}
+__device__ __forceinline__ void store4(float *p, const float4 &v) {
+  *reinterpret_cast<Float4A *>(p) = Float4A{v.x, v.y, v.z, v.w};
+}
+
 template <bool BUF, bool U24>
 struct FeatRows {
   __amdgpu_buffer_rsrc_t rsrc;
@@ -94,7 +107,7 @@ struct FeatRows {
         off = static_cast<uint32_t>(col) * static_cast<uint32_t>(row_bytes) + lane_bytes;
       return __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, static_cast<int>(off), 0, 0));
     } else {
-      return *reinterpret_cast<const float4 *>(base + static_cast<int64_t>(col) * row_bytes + lane_bytes);
+      return load4(reinterpret_cast<const float *>(base + static_cast<int64_t>(col) * row_bytes + lane_bytes));
     }
   }
 };
@@ -187,6 +200,9 @@ __device__ __forceinline__ void spmm_long_runs(const SpmmArgs &a, const FeatRows
   const bool carry = a.accumulate != 0;
   const int f1 = (a.tile_base + tile) * TW + lane;  // the float this lane sums
   const bool adder = wave == 0 && lane < TW && f1 < a.F;
+  // the lane whose four floats the row's end cuts gathers the row's last four floats instead (see the kernel), so
+  // the products of the floats from the last multiple of four on sit 4 - F % 4 slots further right
+  const int slot = lane + ((a.F % 4 != 0 && f1 >= a.F - a.F % 4) ? 4 - a.F % 4 : 0);
   float *const mine = lds + wave * REGION;
   struct StepIds {
     int c[Q];
@@ -262,7 +278,7 @@ __device__ __forceinline__ void spmm_long_runs(const SpmmArgs &a, const FeatRows
 #pragma unroll 8
         for (int t = 0; t < here; ++t) {
           const int w = t / RB, j = t % RB;
-          const float term = lds[w * REGION + (j / NG) * 256 + (j % NG) * TW + lane];
+          const float term = lds[w * REGION + (j / NG) * 256 + (j % NG) * TW + slot];
           if constexpr (RED < 0)
             acc = acc + term;
           else if ((RED == FG_REDUCE_MAX || RED == FG_REDUCE_MIN) && starts && s == 0 && t == 0)
@@ -300,10 +316,15 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(3
   const int tile = static_cast<int>(blockIdx.y) * il + static_cast<int>(blockIdx.x % il);
   const int bx = static_cast<int>(blockIdx.x / il);
   const int gx = static_cast<int>(gridDim.x / il);
-  const int f0 = (a.tile_base + tile) * TW + gl * 4;
-  const bool fok = f0 < a.F;  // F is a multiple of 4: a lane's four floats exist together
+  // A lane owns four adjacent floats.  Where the row ends inside them (feature lengths that are not a multiple of
+  // four) the lane takes the row's LAST four floats instead: it repeats, bit for bit, what its neighbour computes
+  // for the floats they share, and both store the same values.  Lanes wholly past the row only keep the wave's
+  // cross-lane traffic going: they re-read the same last floats and store nothing.
+  const int f0_nominal = (a.tile_base + tile) * TW + gl * 4;
+  const bool fok = f0_nominal < a.F;
+  const int f0 = min(f0_nominal, a.F - 4);
   const int64_t F = a.F;
-  const uint32_t lane_bytes = static_cast<uint32_t>(fok ? f0 : a.F - 4) * 4u;
+  const uint32_t lane_bytes = static_cast<uint32_t>(f0) * 4u;
   const FeatRows<BUF, U24> feat(a.feat, a.n_cols, F);
   const bool carry = a.accumulate != 0;
   // the first workgroups take the long runs (the records come by descending length), one workgroup per run
@@ -370,7 +391,7 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(3
     if constexpr (PICKS)
       if (hi > lo) starts = lo + vo == a.indptr[row];
     if (carry && hi > lo && fok && !starts)
-      acc = *reinterpret_cast<const float4 *>(a.out + static_cast<int64_t>(row) * F + f0);
+      acc = load4(a.out + static_cast<int64_t>(row) * F + f0);
   };
 
   int lo_a, hi_a, row_a, vo_a, lo_b, hi_b, row_b, vo_b;
@@ -431,7 +452,7 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(3
     }
     if (!next_asked) first_ids(lo_b, hi_b, row_b, vo_b, st_b, ids_b, acc_b);  // no group had a nonzero here
     if (fok && row_a >= 0 && (hi_a > lo_a || !carry))
-      *reinterpret_cast<float4 *>(a.out + static_cast<int64_t>(row_a) * F + f0) = acc_a;
+      store4(a.out + static_cast<int64_t>(row_a) * F + f0, acc_a);
 
     lo_a = lo_b;
     hi_a = hi_b;

@@ -71,9 +71,10 @@ def test_column_block_passes_fold_in_the_same_order(msg, reduce):
     adj.data = (adj.data + np.float32(0.25)).astype(np.float32)
     try:
         _lib.config_set("spmm.blocked", 1)
-        # 72 floats: a whole 64-float tile and a partial one; 24: one partial 32-float tile.  Both kernels: the
-        # several-rows-per-wave one (also one wave per run of 512 nonzeros and more) and the row-slot one.
-        for F, multi in ((72, -1), (72, 0), (24, -1)):
+        # 72 floats: a whole 64-float tile and a partial one; 24: one partial 32-float tile; 70 and 30: the row's
+        # end cuts a lane's four floats.  Both kernels: the several-rows-per-wave one (also one workgroup per run
+        # of 1024 nonzeros and more) and the row-slot one.
+        for F, multi in ((72, -1), (72, 0), (24, -1), (70, -1), (30, -1)):
             feat = datasets.spmm_operands(adj, F)
             feat[adj.indices[adj.indptr[7]]] = np.nan         # first message of row 7 (and wherever else the vertex occurs)
             feat[adj.indices[adj.indptr[9] + 3]] = np.nan     # a later message of row 9

@@ -287,7 +287,7 @@ def test_rows_per_wave_kernel_gives_the_same_bits(config_guard, blocks, long_run
     _lib.config_set("spmm.block_cols", blocks[1])
     _lib.config_set("spmm.multi_long", long_run)       # 8: nearly every run takes the one-workgroup-per-run path; 2^20: none
     module = VanillaSpMMhip(adj)
-    for F in (4, 8, 16, 20, 32, 36, 64, 68, 200, 512):
+    for F in (4, 5, 7, 8, 16, 20, 30, 31, 32, 36, 63, 64, 68, 70, 101, 127, 200, 250, 512):
         feat = datasets.spmm_operands(adj, F)
         text = _describe(module, feat)
         assert "rows-per-wave" in text and (("column blocks of %d" % blocks[1]) in text) == bool(blocks[0])
@@ -300,7 +300,10 @@ def test_rows_per_wave_kernel_gives_the_same_bits(config_guard, blocks, long_run
 def test_rows_per_wave_kernel_only_where_it_applies(config_guard, adj_127x255):
     module = VanillaSpMMhip(adj_127x255)
     assert "rows-per-wave" in _describe(module, np.empty((255, 64), np.float32))
-    assert "rows-per-wave" not in _describe(module, np.empty((255, 30), np.float32))       # not a multiple of 4 floats
+    assert "rows-per-wave" in _describe(module, np.empty((255, 30), np.float32))           # the row's end cuts a lane's four floats
+    assert "rows-per-wave" in _describe(module, np.empty((255, 70), np.float32))           # ... in the second tile
+    for F in (3, 66, 129):                             # fewer than four floats in all / in the last tile
+        assert "rows-per-wave" not in _describe(module, np.empty((255, F), np.float32))
     assert "rows-per-wave" not in module.lower_to_ir([placeholder((255, 64))], {"num_feat_partitions": 2}, {})
     _lib.config_set("spmm.lpr", 64)                    # an explicit launch shape asks for the other kernels
     assert "rows-per-wave" not in _describe(module, np.empty((255, 64), np.float32))
