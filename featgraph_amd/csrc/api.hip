@@ -901,7 +901,8 @@ static int sddmm_rows_max_wide(const fg_sddmm_plan *plan) {
 static bool sddmm_use_row_runs(const fg_sddmm_plan *plan, const float *src, const float *dst, int32_t H, int32_t D) {
   const int mode = fg::config().sddmm_rows;
   if (!plan->rows || !plan->rows->seg || mode == 0) return false;
-  if (H != 1 || D % 4 != 0 || !fg::aligned_to(src, 16) || !fg::aligned_to(dst, 16)) return false;
+  // any feature length from four floats on: a lane's piece that the row's end cuts is moved back and masked
+  if (H != 1 || D < 4 || !fg::aligned_to(src, 4) || !fg::aligned_to(dst, 4)) return false;
   if (mode > 0) return true;
   if (plan->rows->n_blocks < 2) return false;  // whole rows: the edge-list kernels take it
   if (plan->force_blocks) return true;

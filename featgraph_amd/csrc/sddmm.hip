@@ -137,7 +137,12 @@ struct VertexRows {
       const uint32_t at = static_cast<uint32_t>(vertex) * row_bytes + off;
       return __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, static_cast<int>(at), 0, 0));
     } else {
-      return *reinterpret_cast<const float4 *>(base + static_cast<int64_t>(vertex) * row_bytes + off);
+      // rows whose length is not a multiple of four floats start at 4-byte aligned addresses only
+      struct alignas(4) Float4A {
+        float x, y, z, w;
+      };
+      const Float4A q = *reinterpret_cast<const Float4A *>(base + static_cast<int64_t>(vertex) * row_bytes + off);
+      return make_float4(q.x, q.y, q.z, q.w);
     }
   }
 };
@@ -265,8 +270,11 @@ __device__ __forceinline__ void rows_wave_place(const RowsArgs &a, int &pass, in
 }
 
 // G: lanes per dot product; NT: 16-byte pieces per lane, 64 floats apart (a tile is 4 * G * NT floats; NT > 1
-// needs G = 16); R: rounds whose gathers are issued together.
-template <bool ACC, bool BUF, int R, int G, int NT>
+// needs G = 16); R: rounds whose gathers are issued together.  CUT: the tile's valid floats are not a multiple of
+// four, so its end cuts some lane's piece: that lane reads the four floats that END at the tile's end instead
+// (they may begin in the tile before; the feature row has at least four floats) and leaves the leading ones,
+// which belong to its neighbour, out of its sum.
+template <bool ACC, bool BUF, int R, int G, int NT, bool CUT>
 __global__ __launch_bounds__(kBlockThreads) void sddmm_rows_kernel(const RowsArgs a) {
   static_assert(NT == 1 || G == 16, "a wide tile is made of whole 64-float pieces");
   constexpr int NG = kWaveSize / G;  // edges per round
@@ -285,11 +293,15 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_rows_kernel(const RowsArg
   // piece k of this lane covers floats first + 64 k + 4 gl ..; lanes past the tile's end re-read its last
   // four floats and contribute zero
   bool kok[NT];
+  int skip[NT];  // leading floats of the piece that are not this lane's (CUT)
   uint32_t lane_bytes[NT];
 #pragma unroll
   for (int k = 0; k < NT; ++k) {
-    kok[k] = k * 64 + gl * 4 < a.valid;
-    lane_bytes[k] = static_cast<uint32_t>(a.first + (kok[k] ? k * 64 + gl * 4 : a.valid - 4)) * 4u;
+    const int start = k * 64 + gl * 4;
+    kok[k] = start < a.valid;
+    const int from = kok[k] ? min(start, a.valid - 4) : a.valid - 4;
+    skip[k] = start - from;
+    lane_bytes[k] = static_cast<uint32_t>(a.first + from) * 4u;
   }
   const int gather_from = G * (lane % NG) + lane / NG;  // lane holding the result of edge offset `lane`
 
@@ -360,10 +372,17 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_rows_kernel(const RowsArg
 #pragma unroll
           for (int k = 0; k < NT; ++k) {
             float q = 0.0f;
-            q = __builtin_fmaf(x[r][k].x, y_a[k].x, q);
-            q = __builtin_fmaf(x[r][k].y, y_a[k].y, q);
-            q = __builtin_fmaf(x[r][k].z, y_a[k].z, q);
-            q = __builtin_fmaf(x[r][k].w, y_a[k].w, q);
+            if constexpr (CUT) {
+              q = skip[k] > 0 ? q : __builtin_fmaf(x[r][k].x, y_a[k].x, q);
+              q = skip[k] > 1 ? q : __builtin_fmaf(x[r][k].y, y_a[k].y, q);
+              q = skip[k] > 2 ? q : __builtin_fmaf(x[r][k].z, y_a[k].z, q);
+              q = __builtin_fmaf(x[r][k].w, y_a[k].w, q);
+            } else {
+              q = __builtin_fmaf(x[r][k].x, y_a[k].x, q);
+              q = __builtin_fmaf(x[r][k].y, y_a[k].y, q);
+              q = __builtin_fmaf(x[r][k].z, y_a[k].z, q);
+              q = __builtin_fmaf(x[r][k].w, y_a[k].w, q);
+            }
             p += kok[k] ? q : 0.0f;
           }
           p = group_sum<G>(p);
@@ -616,20 +635,28 @@ int sddmm_tile_launch(const int32_t *row_p, const int32_t *col_p, const int32_t 
   return tile == 0 ? launch_fast_mode<16, 1, false, 1>(f, stream) : launch_fast_mode<16, 1, false, 2>(f, stream);
 }
 
-template <int G, int NT>
-static void rows_dispatch(const RowsArgs &a, bool acc, bool buf, dim3 grid, hipStream_t stream) {
+template <int G, int NT, bool CUT>
+static void rows_dispatch_cut(const RowsArgs &a, bool acc, bool buf, dim3 grid, hipStream_t stream) {
   constexpr int R = NT == 2 ? 1 : 2;  // rounds per batch: four 16-byte gathers in flight per lane, two batches
   if (!acc) {
     if (buf)
-      sddmm_rows_kernel<false, true, R, G, NT><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+      sddmm_rows_kernel<false, true, R, G, NT, CUT><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
     else
-      sddmm_rows_kernel<false, false, R, G, NT><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+      sddmm_rows_kernel<false, false, R, G, NT, CUT><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
   } else {
     if (buf)
-      sddmm_rows_kernel<true, true, R, G, NT><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+      sddmm_rows_kernel<true, true, R, G, NT, CUT><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
     else
-      sddmm_rows_kernel<true, false, R, G, NT><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+      sddmm_rows_kernel<true, false, R, G, NT, CUT><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
   }
+}
+
+template <int G, int NT>
+static void rows_dispatch(const RowsArgs &a, bool acc, bool buf, dim3 grid, hipStream_t stream) {
+  if (a.valid % 4 != 0)
+    rows_dispatch_cut<G, NT, true>(a, acc, buf, grid, stream);
+  else
+    rows_dispatch_cut<G, NT, false>(a, acc, buf, grid, stream);
 }
 
 // Width of the (first) tile: the whole row when it is short (then fewer lanes share a dot product), else 64

@@ -177,10 +177,14 @@ def test_column_blocked_falls_back_for_odd_lengths_and_heads(config_guard):
     _lib.config_set("sddmm.blocked", 1)
     _lib.config_set("sddmm.block_cols", 500)
     coo = datasets.config_graph("c2-mini").tocoo()
-    src, dst = datasets.sddmm_operands(coo, 30)
-    module = VanillaSDDMMhip(coo)
-    assert "column blocks" not in module.lower_to_ir([placeholder(src.shape), placeholder(dst.shape)], {}, {})
-    np.testing.assert_allclose(_run_sddmm(coo, src, dst), ref.sddmm_x86(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
+    for F, blocked in ((3, False), (30, False), (30, True)):         # below four floats no blocked kernel applies;
+        _lib.config_set("sddmm.rows", -1 if blocked else 0)          # at 30 the row-run kernel does, the re-ordered
+        src, dst = datasets.sddmm_operands(coo, F)                    # edge list (rows = 0) does not
+        module = VanillaSDDMMhip(coo)
+        text = module.lower_to_ir([placeholder(src.shape), placeholder(dst.shape)], {}, {})
+        assert ("column blocks" in text) == (blocked and F >= 4)
+        np.testing.assert_allclose(_run_sddmm(coo, src, dst), ref.sddmm_x86(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
+    _lib.config_set("sddmm.rows", -1)
     src, dst = datasets.sddmm_operands(coo, (4, 16))
     out = _run_sddmm(coo, src, dst, cls=MultiHeadSDDMMhip)
     np.testing.assert_allclose(out, ref.sddmm_mh(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
@@ -238,6 +242,29 @@ def test_row_runs_of_a_row_sorted_list(config_guard, F):
     module = VanillaSDDMMhip(coo)
     assert "column-blocked edge list" in _describe(module, src, dst)
     assert np.array_equal(_run_sddmm(coo, src, dst), outs[0])
+
+
+@pytest.mark.parametrize("F", [5, 6, 7, 30, 31, 62, 63, 65, 66, 70, 127, 129, 130, 131, 250, 258])
+def test_row_runs_when_the_row_end_cuts_a_lanes_piece(config_guard, F):
+    """Feature lengths that are not a multiple of four floats: the lane whose 16-byte piece the row's end cuts reads
+    the four floats that end there and leaves its neighbour's floats out of its sum (also when only one to three
+    floats are left for the last tile, where that piece begins in the tile before).  Small integers make every
+    summation order exact, so a float counted twice or left out shows as a wrong integer."""
+    coo = datasets.config_graph("c2-mini").tocoo()
+    src, dst = datasets.sddmm_operands(coo, F)
+    _lib.config_set("sddmm.blocked", 1)
+    for block_cols, wide in ((700, 1), (700, 2), (64, 2)):
+        _lib.config_set("sddmm.block_cols", block_cols)
+        _lib.config_set("sddmm.rows_wide", wide)
+        module = VanillaSDDMMhip(coo)
+        assert "row runs" in _describe(module, src, dst)
+        module.build([placeholder(src.shape), placeholder(dst.shape)], {}, {})
+        module.out_tvm.tensor.fill_(7.0)
+        out = module.run([nd.array(src, module.ctx), nd.array(dst, module.ctx)]).asnumpy()
+        np.testing.assert_allclose(out, ref.sddmm_f64(coo.row, coo.col, src, dst), rtol=RTOL, atol=ATOL)
+        isrc, idst = np.rint(src * 2), np.rint(dst * 2)
+        got = module.run([nd.array(isrc, module.ctx), nd.array(idst, module.ctx)]).asnumpy()
+        assert np.array_equal(got, ref.sddmm_f64(coo.row, coo.col, isrc, idst).astype(np.float32))
 
 
 @pytest.mark.parametrize("F", [128, 132, 192, 200, 260, 512])
@@ -307,9 +334,12 @@ def test_which_lists_take_the_row_run_kernel(config_guard):
     inv = np.empty_like(order)
     inv[order] = np.arange(coo.nnz)
     assert np.array_equal(_run_sddmm(ragged, src, dst)[inv], base)
-    # 30 floats or several heads: neither blocked kernel applies
+    # 30 floats: the row's end cuts a lane's piece, which the row-run kernel moves back and masks; below four
+    # floats it does not apply
     src30, dst30 = datasets.sddmm_operands(coo, 30)
-    assert "row runs" not in _describe(VanillaSDDMMhip(coo), src30, dst30)
+    assert "row runs" in _describe(VanillaSDDMMhip(coo), src30, dst30)
+    src3, dst3 = datasets.sddmm_operands(coo, 3)
+    assert "row runs" not in _describe(VanillaSDDMMhip(coo), src3, dst3)
 
 
 @pytest.mark.parametrize("F,block_cols", [(64, 500), (32, 300), (256, 700), (64, 1000)])
