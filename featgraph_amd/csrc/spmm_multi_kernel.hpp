@@ -181,7 +181,7 @@ struct alignas(4) Float4U {
 // of four waves x kLongRounds rounds proceed at once, and only the adds stay ordered: the products go through LDS
 // to the first 4*G lanes of the first wave, lane i of which owns float i of the tile and adds its terms one by
 // one, the waves' regions in turn.  Same terms, same order, same roundings as everywhere else.
-constexpr int kLongRounds = 8;  // rounds per wave and step; the gathers of two steps are in flight per wave
+constexpr int kLongRounds = 8;  // rounds per wave and step
 
 template <int G, bool BUF, bool U24, int RED, int MSG>
 __device__ __forceinline__ void spmm_long_runs(const SpmmArgs &a, const FeatRows<BUF, U24> &feat, int first_run,
@@ -260,18 +260,18 @@ __device__ __forceinline__ void spmm_long_runs(const SpmmArgs &a, const FeatRows
     auto count = [&](int s) { return max(0, min(RB, len - at(s))); };
 
     const int n_steps = (len + SB - 1) / SB;
-    float4 xa[R], xb[R];
+    float4 x[R];
     StepIds ids_cur, ids_nxt;
     load_ids(0, ids_cur);
-    issue(xa, ids_cur, count(0));
+    issue(x, ids_cur, count(0));
     load_ids(1, ids_nxt);
-    // One step: the next step's gathers go out first, then this step's products go to LDS, the first wave adds
-    // them in order, and the regions are free again.  Every wave passes both barriers of every step.
-    auto step = [&](int s, float4(&cur)[R], float4(&nxt)[R]) {
-      issue(nxt, ids_nxt, count(s + 1));
+    // One step: this step's products go to LDS, the next step's gathers go out into the registers they leave,
+    // the first wave adds the products in order, and the regions are free again.  Every wave passes both barriers.
+    for (int s = 0; s < n_steps; ++s) {
       StepIds ids_after;
       load_ids(s + 2, ids_after);
-      products(cur, ids_cur, count(s));
+      products(x, ids_cur, count(s));
+      issue(x, ids_nxt, count(s + 1));
       __syncthreads();
       if (wave == 0 && lane < TW) {
         const int here = min(SB, len - s * SB);
@@ -290,10 +290,6 @@ __device__ __forceinline__ void spmm_long_runs(const SpmmArgs &a, const FeatRows
       __syncthreads();
       ids_cur = ids_nxt;
       ids_nxt = ids_after;
-    };
-    for (int s = 0; s < n_steps; s += 2) {
-      step(s, xa, xb);
-      if (s + 1 < n_steps) step(s + 1, xb, xa);
     }
     if (adder) a.out[static_cast<int64_t>(row) * F + f1] = acc;
   }
