@@ -208,13 +208,18 @@ def main():
     ap.add_argument("--feat-len", type=int, default=64, help="feature length of the timed step")
     ap.add_argument("--graph", default="c2", help="named synthetic configuration (featgraph_amd.datasets.CONFIGS)")
     ap.add_argument("--only", choices=["all", "spmm", "sddmm", "sddmm_shuffled", "copy", "mh_sddmm", "mh_spmm", "mh_sddmm_softmax",
-                                       "mh_attention", "mh_attention_kv", "gather_probe", "gather_store_probe"],
+                                       "mh_attention", "mh_attention_kv", "mh_attention_grad", "gather_probe", "gather_store_probe"],
                     default="all",
                     help="spmm / sddmm / copy / gather_probe: run just that kernel (for profiler runs), no sweep, no "
                          "CPU leg; mh_sddmm / mh_spmm: the multi-head operators (8 heads of --feat-len floats, use "
                          "--graph c4)")
     ap.add_argument("--band-rows", type=int, default=0,
                     help="with --only gather_probe: rows per band (default 16384 rows of a 64-float tile)")
+    ap.add_argument("--fold-cols", type=int, default=0,
+                    help="with --only spmm / sddmm: column ids taken modulo this (the same rows and nonzeros over a "
+                         "feature matrix of so many rows; 8192 rows of 64 floats fit one L2, so every gather hits)")
+    ap.add_argument("--degree-cap", type=int, default=0,
+                    help="with --only spmm / sddmm: every row cut to at most so many nonzeros (takes the hub rows out)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg and the parity checks")
     ap.add_argument("--no-sweep", action="store_true", help="skip the feature-length sweep")
     ap.add_argument("--no-mh", action="store_true", help="skip the multi-head operators on the 2.45M-vertex graph")
@@ -226,8 +231,9 @@ def main():
     import numpy as np
     import torch
     from featgraph_amd import _lib, datasets, nd, placeholder
-    from featgraph_amd.module import (EdgeSoftmaxhip, GeneralizedSpMMhip, MultiHeadAttentionhip, MultiHeadSDDMMhip,
-                                      MultiHeadSDDMMSoftmaxhip, MultiHeadSpMMhip, VanillaSDDMMhip, VanillaSpMMhip)
+    from featgraph_amd.module import (EdgeSoftmaxhip, GeneralizedSpMMhip, MultiHeadAttentionGradhip,
+                                      MultiHeadAttentionhip, MultiHeadSDDMMhip, MultiHeadSDDMMSoftmaxhip,
+                                      MultiHeadSpMMhip, VanillaSDDMMhip, VanillaSpMMhip)
 
     L = _lib.lib()  # fail now if the HIP library is missing
     if not torch.cuda.is_available():
@@ -330,6 +336,21 @@ def main():
         args.graph, n_rows, n_cols, nnz, int(np.diff(adj.indptr).max()), datasets.structure_checksum(adj),
         time.time() - t))
     F = args.feat_len
+    if args.only in ("spmm", "sddmm") and (args.fold_cols or args.degree_cap):
+        # diagnostic variants of the graph: what bounds the kernels when the cache misses or the hub rows are taken away
+        import scipy.sparse
+        if args.degree_cap:
+            deg = np.diff(adj.indptr)
+            keep_deg = np.minimum(deg, args.degree_cap)
+            keep = (np.arange(nnz) - np.repeat(adj.indptr[:-1], deg)) < np.repeat(keep_deg, deg)
+            indptr = np.zeros(n_rows + 1, np.int32)
+            np.cumsum(keep_deg, out=indptr[1:])
+            adj = scipy.sparse.csr_matrix((adj.data[keep], adj.indices[keep], indptr), shape=adj.shape)
+        if args.fold_cols:
+            adj = scipy.sparse.csr_matrix((adj.data, (adj.indices % args.fold_cols).astype(np.int32), adj.indptr),
+                                          shape=(n_rows, args.fold_cols))
+        n_rows, n_cols, nnz = adj.shape[0], adj.shape[1], adj.nnz
+        log("variant: %d x %d, nnz %d, max degree %d" % (n_rows, n_cols, nnz, int(np.diff(adj.indptr).max())))
 
     if args.only == "gather_probe":
         feat_t = device_normal((n_cols, F), 1)
@@ -376,6 +397,17 @@ def main():
             op.build([placeholder((n_c, H, D)), placeholder((n_r, H, D))], {}, {})
             ins = [src, dst]
             b, b_min = mh_sddmm_alg_bytes(e, H, D), 8 * e + 4 * H * e + 4 * H * D * (n_r + n_c)
+        elif kind == "mh_attention_grad":
+            # backward of the layer whose key is its value: scores + softmax recomputed, then the softmax gradient,
+            # two multi-head SpMMs over the transposed matrix, one over the matrix and one multi-head SDDMM
+            op = MultiHeadAttentionGradhip(graph_adj)
+            src, dst = device_normal((n_c, H, D), 11 + D), device_normal((n_r, H, D), 12 + D)
+            src *= 0.25
+            ins = [src, dst, device_normal((n_r, H, D), 15 + D)]
+            op.build([placeholder((n_c, H, D)), placeholder((n_r, H, D))], {}, {})
+            b = (2 * mh_sddmm_alg_bytes(e, H, D) + 2 * mh_spmm_alg_bytes(e, n_c, H, D) + mh_spmm_alg_bytes(e, n_r, H, D)
+                 + e * (3 * 4 * H) + 2 * e * (4 + 8 * H) + 3 * 4 * H * D * n_c)
+            b_min = 8 * e + 4 * H * D * (3 * n_r + 3 * n_c)
         elif kind in ("mh_attention", "mh_attention_kv"):
             # scores, softmax and weighted sum in one kernel; "mh_attention": the vertex features are key and value
             shared = kind == "mh_attention"
@@ -405,16 +437,21 @@ def main():
         p = rows_probe(src, e)
         if p and kind == "mh_attention_kv":      # two gathered rows per edge
             p = dict(p, ms=2 * p["ms"], gathers=2 * e)
+        if p and kind == "mh_attention_grad":    # five operators that each gather one row per edge
+            p = dict(p, ms=5 * p["ms"], gathers=5 * e)
+        if kind == "mh_attention_grad":
+            row["flops_note"] = "10 * E * H * D: five gather-and-multiply operators"
         if p:
             row.update({"gather_ceiling_ms": p["ms"], "gather_ceiling_row_TBps": p["row_TBps"],
                         "frac_of_gather_ceiling": p["ms"] / ms})
         tr, tr_src = committed_traffic_mh(kind, D) if graph_adj.shape[0] == 2449029 else (None, None)
         if tr:
             row.update({"traffic": tr, "traffic_source": tr_src, "hbm_frac_traffic": tr / ms / 1e6 / HBM_PEAK_GBPS})
-        row.update({"ms": ms, "GFLOPs": 2.0 * e * H * D / ms / 1e6, "alg_GBps": b / ms / 1e6,
+        row.update({"ms": ms, "GFLOPs": (10.0 if kind == "mh_attention_grad" else 2.0) * e * H * D / ms / 1e6,
+                    "alg_GBps": b / ms / 1e6,
                     "frac": b / ms / 1e6 / HBM_PEAK_GBPS, "hbm_frac_compulsory": b_min / ms / 1e6 / HBM_PEAK_GBPS,
                     "algorithmic_bytes": b, "compulsory_bytes": b_min})
-        if check:
+        if check and kind != "mh_attention_grad":   # (its parity runs at full size in tests/test_full_size.py)
             from oracle import ref
             out = op.out_tvm.asnumpy()
             if kind == "mh_sddmm":
@@ -456,7 +493,7 @@ def main():
                             "gather_store_probe": pw})
         return row
 
-    if args.only in ("mh_sddmm", "mh_spmm", "mh_sddmm_softmax", "mh_attention", "mh_attention_kv"):
+    if args.only in ("mh_sddmm", "mh_spmm", "mh_sddmm_softmax", "mh_attention", "mh_attention_kv", "mh_attention_grad"):
         row = mh_case(args.only, adj, F, args.steps, args.warmup, False)
         row.update({"kernel": args.only, "graph": args.graph})
         print(json.dumps(row))
@@ -499,7 +536,7 @@ def main():
         ins = sddmm_case(sddmm, F)
         ms = timed(lambda: sddmm.run(ins), args.steps, args.warmup)
         b = sddmm_alg_bytes(nnz, F)
-        print(json.dumps({"kernel": args.only, "F": F, "ms": ms, "alg_GBps": b / ms / 1e6,
+        print(json.dumps({"kernel": args.only, "F": F, "nnz": nnz, "n_cols": n_cols, "ms": ms, "alg_GBps": b / ms / 1e6,
                           "frac": b / ms / 1e6 / HBM_PEAK_GBPS, "plan_seconds": plan_seconds["sddmm"]}))
         return
 
@@ -521,7 +558,8 @@ def main():
     roofline = {
         "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
         "traffic": traffic, "traffic_source": traffic_source,
-        "algorithmic_bytes": alg, "kernel": "spmm (CSR, feat-len %d)" % F, "launch_ms": ms,
+        "algorithmic_bytes": alg, "kernel": "spmm_multi_kernel<%d,true,true,-1,0>" % (4 if F <= 16 else 8 if F <= 32 else 16),
+        "launch_ms": ms,
         "compulsory_bytes": b_min, "hbm_frac_compulsory": b_min / ms / 1e6 / HBM_PEAK_GBPS,
         "l2_fabric_frac": (traffic / ms / 1e6 / HBM_PEAK_GBPS) if traffic else None,
         "frac_bounded": (traffic / ms / 1e6 / HBM_PEAK_GBPS) if traffic else None,
@@ -734,6 +772,9 @@ def main():
             "ms": hb["ms"], "algorithmic_bytes": hb["algorithmic_bytes"], "achieved": hb["alg_GBps"],
             "frac": hb["frac"], "traffic": hb.get("traffic"), "frac_traffic": hb.get("hbm_frac_traffic"),
             "parity": (hb.get("parity") or {}).get("bit_exact_vs_cpu_checker")}
+        mh.append(mh_case("mh_attention_grad", big, 64, 3, 1, False))
+        torch.cuda.empty_cache()
+        log("mh_attention_grad D=64 (value = key): %.3f ms" % mh[-1]["ms"])
         result["multi_head"] = {"graph": "c4: %d vertices, %d edges" % (big.shape[0], big.nnz), "rows": mh,
                                 "note": "1.25 - 5 GB of features and mean degree 25: nearly every neighbour gather "
                                         "goes to HBM.  `frac` is algorithmic bytes / time / 8 TB/s (above 1 for SDDMM "

@@ -307,6 +307,37 @@ def test_c4_fused_attention(c4, D, shared):
         assert not out[~has_edges].any()
 
 
+@pytest.mark.parametrize("D,shared", [(16, True), (32, False)])
+def test_c4_attention_backward(c4, D, shared):
+    """All three gradients of the attention layer on the whole 2.45M-vertex graph (multi-head SpMM over the
+    transposed matrix with permuted weights, softmax gradient, multi-head SDDMM), against the composed CPU checker."""
+    from featgraph_amd.module import MultiHeadAttentionGradhip
+    adj = c4
+    n, H = adj.shape[0], 8
+    _say("attention backward c4 H=8 D=%d %s through MultiHeadAttentionGradhip" % (D, "key = value" if shared else "key, value"))
+    module = MultiHeadAttentionGradhip(adj)
+    module.build([placeholder((n, H, D))] * (2 if shared else 3), {}, {})
+    key_dev, key = _device_normal((n, H, D), 1000 + D, module.ctx)
+    key_dev *= 0.25
+    key *= np.float32(0.25)
+    query_dev, query = _device_normal((n, H, D), 1100 + D, module.ctx)
+    dout_dev, dout = _device_normal((n, H, D), 1200 + D, module.ctx)
+    ins, value = [key_dev, query_dev], None
+    if not shared:
+        value_dev, value = _device_normal((n, H, D), 1300 + D, module.ctx)
+        ins.append(value_dev)
+    d_key, d_query, d_value = module.run(ins + [dout_dev])
+    want_key, want_query, want_value = ref.attention_mh_backward(adj.indptr, adj.indices, key, query, value, dout)
+    # sums of up to thousands of float32 terms whose weights come from a float32 softmax: the forward operator's
+    # tolerance scaled to the size of the gradients
+    np.testing.assert_allclose(d_query.asnumpy(), want_query, rtol=1e-3, atol=5e-4)
+    np.testing.assert_allclose(d_key.asnumpy(), want_key, rtol=1e-3, atol=5e-4)
+    if shared:
+        assert d_value is None
+    else:
+        np.testing.assert_allclose(d_value.asnumpy(), want_value, rtol=1e-3, atol=5e-4)
+
+
 def test_benchmark_commands_run_on_a_small_graph(tmp_path, capsys):
     import scipy.sparse
     from featgraph_amd.benchmark import bench_vanilla_sddmm, bench_vanilla_spmm
