@@ -293,6 +293,16 @@ int multi_interleave(int n_tiles) {
   return (il > 1 && n_tiles % il == 0) ? il : 1;
 }
 
+// Feature rows of several 64-float tiles whose rest is 1 .. 32 floats: the rest runs as a tile of 16 or 32 floats
+// (4 or 8 lanes per row, so 16 or 8 rows per wave) over the same records and passes, instead of a 64-float tile
+// with most of its lanes idle (the 232,965-vertex graph at 65 / 72 / 96 floats: 4.1 / 3.4 / 3.4 ms with a 64-float
+// rest tile).  0: no such rest.
+int multi_tail_tile(int32_t F) {
+  if (fg::spmm_multi_tile(F) != 64 || F < 64) return 0;
+  const int rest = F % 64;
+  return rest == 0 || rest > 32 ? 0 : rest <= 16 ? 16 : 32;
+}
+
 int multi_run(const fg_spmm_plan *plan, const fg::MultiRuns *runs, fg::SpmmArgs a, hipStream_t st) {
   if (runs->ids_p) {  // the records index the re-laid ids and say where each run's values start in the CSR array
     a.indices = runs->ids_p;
@@ -305,7 +315,7 @@ int multi_run(const fg_spmm_plan *plan, const fg::MultiRuns *runs, fg::SpmmArgs 
     a.long_runs = runs->long_runs[pass];
     a.long_blocks = std::min(a.long_runs, 2048);  // one workgroup per long run at a time
   };
-  if (runs->passes == 1) {
+  if (runs->passes == 1 && multi_tail_tile(a.F) == 0) {
     a.runs = runs->rec;
     long_split(0);
     a.tile_base = 0;
@@ -318,14 +328,24 @@ int multi_run(const fg_spmm_plan *plan, const fg::MultiRuns *runs, fg::SpmmArgs 
   // tile: workgroups are dispatched tile pair after tile pair, so the resident waves gather from one or two
   // tiles' bands at a time, a pair's tail overlaps the next pair's head, and there are n_tiles times fewer
   // launch boundaries than with a launch per (tile, pass).
-  a.tile_base = 0;
-  a.n_tiles = n_tiles;
-  a.interleave_tiles = multi_interleave(n_tiles);
+  const int tail = multi_tail_tile(a.F);
+  const int main_tiles = tail ? n_tiles - 1 : n_tiles;
   for (int b = 0; b < runs->passes; ++b) {
     a.runs = runs->rec + static_cast<int64_t>(b) * n;
     long_split(b);
     a.accumulate = b > 0;
+    a.multi_tile = 0;
+    a.tile_base = 0;
+    a.n_tiles = main_tiles;
+    a.interleave_tiles = multi_interleave(main_tiles);
     if (int rc = fg::spmm_multi_launch(a, st)) return rc;
+    if (tail) {  // the same pass, the same records, fewer lanes per row
+      a.multi_tile = tail;
+      a.tile_base = main_tiles * (tile / tail);
+      a.n_tiles = 1;
+      a.interleave_tiles = 1;
+      if (int rc = fg::spmm_multi_launch(a, st)) return rc;
+    }
   }
   return FG_OK;
 }
@@ -1099,11 +1119,18 @@ int fg_spmm_describe(const fg_spmm_plan *plan, int32_t H, int32_t D, int32_t fea
     const int tile = fg::spmm_multi_tile(a.F);
     const int n_tiles = (a.F + tile - 1) / tile;
     const int n_passes = runs->passes, merge = runs->merge;
-    char passes[144] = "1 launch";
+    const int tail = multi_tail_tile(a.F);
+    const int main_tiles = tail ? n_tiles - 1 : n_tiles;
+    char rest[96] = "";
+    if (tail) snprintf(rest, sizeof(rest), ", the rest of the row as a tile of %d floats in a launch of its own", tail);
+    char passes[288] = "1 launch";
     if (n_passes > 1)
-      snprintf(passes, sizeof(passes), "%d launches (one per column block: %d column blocks of %d, each over %d tiles, %d in turn)",
-               n_passes, n_passes, static_cast<int>(std::min<int64_t>(int64_t{plan->block_cols} * merge, 0x7fffffff)),
-               n_tiles, multi_interleave(n_tiles));
+      snprintf(passes, sizeof(passes), "%d launches (one per column block: %d column blocks of %d, each over %d tiles, %d in turn%s)",
+               n_passes * (tail ? 2 : 1), n_passes,
+               static_cast<int>(std::min<int64_t>(int64_t{plan->block_cols} * merge, 0x7fffffff)), main_tiles,
+               multi_interleave(main_tiles), rest);
+    else if (tail)
+      snprintf(passes, sizeof(passes), "2 launches (%d tiles%s)", main_tiles, rest);
     snprintf(buf, static_cast<size_t>(cap),
              "spmm_csr rows=%lld cols=%lld nnz=%lld max_degree=%d H=%d D=%d | kernel=rows-per-wave(pipelined) "
              "floats/lane=4 lanes/row=%d rows/wave=%d tile=%d floats x %d tiles gathers-in-flight=%d "

@@ -69,6 +69,7 @@ struct SpmmArgs {
   int32_t long_runs = 0;    // the first long_runs records are long runs: one workgroup each, in the first
   int32_t long_blocks = 0;  // long_blocks workgroups of the grid
   int32_t interleave_tiles = 1;  // this many tiles alternate workgroup by workgroup along grid.x; the rest along grid.y
+  int32_t multi_tile = 0;        // floats per tile of the several-rows-per-wave kernel (16 / 32 / 64); 0: by feature length
   // records over a re-laid copy of the ids (MultiRuns::ids_p): `indices` is that copy, and a run's values start
   // at the CSR position in the record's fourth entry
   int32_t vals_by_csr = 0;

@@ -189,11 +189,9 @@ int multi_runs_build(const int32_t *seg, const int32_t *row_order, const int32_t
 }
 
 bool spmm_multi_applies(const SpmmArgs &a) {
-  // Any feature length from four floats on whose last tile holds none or at least four floats (a lane that the
-  // row's end cuts takes the row's last four floats, which must lie in its own tile); rows that are not 16-byte
-  // aligned are read with 4-byte aligned accesses.
-  const int rest = a.F % spmm_multi_tile(a.F);
-  return a.H == 1 && a.F >= 4 && (rest == 0 || rest >= 4) && aligned_to(a.feat, 4) && aligned_to(a.out, 4);
+  // Any feature length from four floats on (a lane that the row's end cuts takes the row's last four floats and
+  // stores only its own); rows that are not 16-byte aligned are read with 4-byte aligned accesses.
+  return a.H == 1 && a.F >= 4 && aligned_to(a.feat, 4) && aligned_to(a.out, 4);
 }
 
 bool spmm_multi_general_applies(const SpmmArgs &a) {
@@ -213,7 +211,7 @@ int spmm_multi_launch(const SpmmArgs &a, hipStream_t stream) {
     return fail(FG_EINVAL, "inconsistent long-run split (%d runs, %d workgroups)", a.long_runs, a.long_blocks);
   const bool buf = static_cast<int64_t>(a.n_cols) * a.F * 4 < (int64_t{1} << 32) && config().spmm_buffer_loads != 0;
   const bool u24 = a.n_cols <= (1 << 24) && static_cast<int64_t>(a.F) * 4 < (1 << 24);
-  const int tile = spmm_multi_tile(a.F);
+  const int tile = a.multi_tile ? a.multi_tile : spmm_multi_tile(a.F);
   if (a.reduce >= 0) {
     if (!spmm_multi_general_applies(a))
       return fail(FG_EINVAL, "the generalised several-rows-per-wave kernel does not take this call");

@@ -86,6 +86,12 @@ __device__ __forceinline__ float4 load4(const float *p) {
 __device__ __forceinline__ void store4(float *p, const float4 &v) {
   *reinterpret_cast<Float4A *>(p) = Float4A{v.x, v.y, v.z, v.w};
 }
+// The same without the first `skip` floats (1 .. 3), which belong to another lane.
+__device__ __forceinline__ void store4_from(float *p, const float4 &v, int skip) {
+  if (skip <= 1) p[1] = v.y;
+  if (skip <= 2) p[2] = v.z;
+  p[3] = v.w;
+}
 
 template <bool BUF, bool U24>
 struct FeatRows {
@@ -314,11 +320,13 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(3
   const int gx = static_cast<int>(gridDim.x / il);
   // A lane owns four adjacent floats.  Where the row ends inside them (feature lengths that are not a multiple of
   // four) the lane takes the row's LAST four floats instead: it repeats, bit for bit, what its neighbour computes
-  // for the floats they share, and both store the same values.  Lanes wholly past the row only keep the wave's
-  // cross-lane traffic going: they re-read the same last floats and store nothing.
+  // for the floats they share, and stores only its own (the shared ones may lie in the tile before, whose carried
+  // sums another wave updates in the same launch).  Lanes wholly past the row only keep the wave's cross-lane
+  // traffic going: they re-read the same last floats and store nothing.
   const int f0_nominal = (a.tile_base + tile) * TW + gl * 4;
   const bool fok = f0_nominal < a.F;
   const int f0 = min(f0_nominal, a.F - 4);
+  const int shared = f0_nominal - f0;  // leading floats of the lane's four that are its neighbour's
   const int64_t F = a.F;
   const uint32_t lane_bytes = static_cast<uint32_t>(f0) * 4u;
   const FeatRows<BUF, U24> feat(a.feat, a.n_cols, F);
@@ -447,8 +455,13 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(3
       rem -= B;
     }
     if (!next_asked) first_ids(lo_b, hi_b, row_b, vo_b, st_b, ids_b, acc_b);  // no group had a nonzero here
-    if (fok && row_a >= 0 && (hi_a > lo_a || !carry))
-      store4(a.out + static_cast<int64_t>(row_a) * F + f0, acc_a);
+    if (fok && row_a >= 0 && (hi_a > lo_a || !carry)) {
+      float *const to = a.out + static_cast<int64_t>(row_a) * F + f0;
+      if (shared == 0)
+        store4(to, acc_a);
+      else
+        store4_from(to, acc_a, shared);
+    }
 
     lo_a = lo_b;
     hi_a = hi_b;
@@ -490,8 +503,9 @@ int launch_multi(const SpmmArgs &a, int64_t blocks, bool buf, bool u24, hipStrea
 // The generalised operator with message MSG and reducer RED, tile width by feature length as for the plain one.
 template <int RED, int MSG>
 int launch_multi_general_tile(const SpmmArgs &a, int64_t blocks, hipStream_t stream) {
-  if (a.F <= 16) return launch_multi<4, RED, MSG>(a, blocks, true, true, stream);
-  if (a.F <= 32) return launch_multi<8, RED, MSG>(a, blocks, true, true, stream);
+  const int tile = a.multi_tile ? a.multi_tile : spmm_multi_tile(a.F);
+  if (tile == 16) return launch_multi<4, RED, MSG>(a, blocks, true, true, stream);
+  if (tile == 32) return launch_multi<8, RED, MSG>(a, blocks, true, true, stream);
   return launch_multi<16, RED, MSG>(a, blocks, true, true, stream);
 }
 

@@ -287,7 +287,9 @@ def test_rows_per_wave_kernel_gives_the_same_bits(config_guard, blocks, long_run
     _lib.config_set("spmm.block_cols", blocks[1])
     _lib.config_set("spmm.multi_long", long_run)       # 8: nearly every run takes the one-workgroup-per-run path; 2^20: none
     module = VanillaSpMMhip(adj)
-    for F in (4, 5, 7, 8, 16, 20, 30, 31, 32, 36, 63, 64, 68, 70, 101, 127, 200, 250, 512):
+    # 17, 33, 65 .. 67, 129 .. 131, 193: the last tile holds one to three floats only; 68 .. 96, 200, 602: a rest of up to 32
+    # floats behind whole 64-float tiles runs as a narrower tile in launches of its own
+    for F in (4, 5, 7, 8, 16, 17, 20, 30, 31, 32, 33, 36, 63, 64, 65, 66, 67, 68, 70, 90, 96, 101, 127, 129, 130, 131, 193, 200, 250, 512, 602):
         feat = datasets.spmm_operands(adj, F)
         text = _describe(module, feat)
         assert "rows-per-wave" in text and (("column blocks of %d" % blocks[1]) in text) == bool(blocks[0])
@@ -302,8 +304,9 @@ def test_rows_per_wave_kernel_only_where_it_applies(config_guard, adj_127x255):
     assert "rows-per-wave" in _describe(module, np.empty((255, 64), np.float32))
     assert "rows-per-wave" in _describe(module, np.empty((255, 30), np.float32))           # the row's end cuts a lane's four floats
     assert "rows-per-wave" in _describe(module, np.empty((255, 70), np.float32))           # ... in the second tile
-    for F in (3, 66, 129):                             # fewer than four floats in all / in the last tile
-        assert "rows-per-wave" not in _describe(module, np.empty((255, F), np.float32))
+    for F in (66, 129):                                # ... and reaches back into the tile before
+        assert "rows-per-wave" in _describe(module, np.empty((255, F), np.float32))
+    assert "rows-per-wave" not in _describe(module, np.empty((255, 3), np.float32))        # fewer than four floats in all
     assert "rows-per-wave" not in module.lower_to_ir([placeholder((255, 64))], {"num_feat_partitions": 2}, {})
     _lib.config_set("spmm.lpr", 64)                    # an explicit launch shape asks for the other kernels
     assert "rows-per-wave" not in _describe(module, np.empty((255, 64), np.float32))
@@ -566,8 +569,9 @@ def test_tiles_of_one_launch_in_turn_or_one_after_the_other(config_guard, interl
     feat = datasets.spmm_operands(adj, F)
     module = VanillaSpMMhip(adj)
     text = module.lower_to_ir([placeholder(feat.shape)], {}, {})
-    n_tiles = (F + 63) // 64
+    n_tiles = F // 64 + (F % 64 > 32)                  # a rest of up to 32 floats runs as a narrower tile of its own
     assert "rows-per-wave" in text and "%d in turn" % (interleave if n_tiles % interleave == 0 else 1) in text
+    assert ("the rest of the row as a tile of 16 floats" in text) == (F == 260)
     module.build([placeholder(feat.shape)], {}, {})
     module.out_tvm.tensor.fill_(4.0)
     assert np.array_equal(module.run([nd.array(feat, module.ctx)]).asnumpy(), _oracle(adj, feat))
