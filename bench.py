@@ -218,6 +218,10 @@ def main():
     ap.add_argument("--fold-cols", type=int, default=0,
                     help="with --only spmm / sddmm: column ids taken modulo this (the same rows and nonzeros over a "
                          "feature matrix of so many rows; 8192 rows of 64 floats fit one L2, so every gather hits)")
+    ap.add_argument("--squeeze-cols", default="",
+                    help="with --only spmm / sddmm: W:K maps the column ids of every band of W columns onto the band's "
+                         "first K columns, ascending order kept (same passes, same runs, a smaller gather target per "
+                         "pass: W = the pass width that lower_to_ir reports, K = 8192 rows of 64 floats fit one L2)")
     ap.add_argument("--degree-cap", type=int, default=0,
                     help="with --only spmm / sddmm: every row cut to at most so many nonzeros (takes the hub rows out)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg and the parity checks")
@@ -336,7 +340,7 @@ def main():
         args.graph, n_rows, n_cols, nnz, int(np.diff(adj.indptr).max()), datasets.structure_checksum(adj),
         time.time() - t))
     F = args.feat_len
-    if args.only in ("spmm", "sddmm") and (args.fold_cols or args.degree_cap):
+    if args.only in ("spmm", "sddmm") and (args.fold_cols or args.degree_cap or args.squeeze_cols):
         # diagnostic variants of the graph: what bounds the kernels when the cache misses or the hub rows are taken away
         import scipy.sparse
         if args.degree_cap:
@@ -349,6 +353,11 @@ def main():
         if args.fold_cols:
             adj = scipy.sparse.csr_matrix((adj.data, (adj.indices % args.fold_cols).astype(np.int32), adj.indptr),
                                           shape=(n_rows, args.fold_cols))
+        if args.squeeze_cols:
+            width, kept = (int(x) for x in args.squeeze_cols.split(":"))
+            band, inside = np.divmod(adj.indices.astype(np.int64), width)
+            adj = scipy.sparse.csr_matrix((adj.data, (band * width + inside * kept // width).astype(np.int32), adj.indptr),
+                                          shape=adj.shape)
         n_rows, n_cols, nnz = adj.shape[0], adj.shape[1], adj.nnz
         log("variant: %d x %d, nnz %d, max degree %d" % (n_rows, n_cols, nnz, int(np.diff(adj.indptr).max())))
 
