@@ -270,6 +270,14 @@ FG_API int fg_sddmm_coo_general_plan_f32(const fg_sddmm_plan *plan, const float 
  * and out are [nnz, H] and may be the same buffer.  A score of -inf is a masked
  * edge: weight 0 wherever it stands in the row; a row and head with nothing
  * but -inf gives NaN (0 / 0), as the textbook softmax does.
+ * Accuracy: float32 throughout, with the device library's expf (documented to
+ * 1 ulp).  A weight of this entry point is one expf and one division over a
+ * sum of such terms: within rtol 1e-5 of the exact softmax of the float32
+ * scores.  The fused entry points below (fg_sddmm_softmax_plan_f32,
+ * fg_attention_csr_mh_f32) keep a running maximum and rescale their partial
+ * sums by a further expf whenever it grows, and compute the scores in the same
+ * kernel, whose float32 rounding enters the exponent: they are held to
+ * rtol 5e-5 and 1e-4.
  */
 FG_API int fg_edge_softmax_csr_f32(int64_t n_rows, const int32_t *indptr, const float *scores, float *out, int32_t H,
                                    void *stream);

@@ -9,7 +9,7 @@ import pytest
 import scipy.sparse
 
 from featgraph_amd import _lib, datasets, nd, placeholder
-from featgraph_amd.module import MultiHeadAttentionhip
+from featgraph_amd.module import EdgeSoftmaxhip, MultiHeadAttentionhip, MultiHeadSDDMMhip, MultiHeadSpMMhip
 from oracle import ref
 
 pytestmark = pytest.mark.gpu
@@ -116,3 +116,24 @@ def test_attention_grid_of_a_few_workgroups_and_errors_through_the_c_abi():
         module.build([placeholder(key.shape), placeholder((query.shape[0] + 1,) + query.shape[1:])], {}, {})
     with pytest.raises(ValueError):
         module.build([placeholder(key.shape), placeholder(query.shape), placeholder((key.shape[0], 8, 32))], {}, {})
+
+
+@pytest.mark.parametrize("H,D", [(8, 64), (8, 16), (4, 32)])
+def test_the_three_operators_one_after_the_other_meet_the_tighter_bar(H, D):
+    """Multi-head SDDMM, the standalone edge softmax and multi-head SpMM run one after the other: no running maximum
+    is rescaled and every weight is one expf and one division, so the chain meets rtol 1e-5 (atol 1e-5 on outputs of
+    magnitude ~1) where the fused kernels are held to 1e-4."""
+    adj = datasets.config_graph("c4-mini")
+    key, query, _ = _operands(adj, H, D, seed=7 * H + D)
+    coo = adj.tocoo()                                     # row-sorted, the CSR order
+    scores = MultiHeadSDDMMhip(coo)
+    scores.build([placeholder(key.shape), placeholder(query.shape)], {}, {})
+    s = scores.run([nd.array(key, scores.ctx), nd.array(query, scores.ctx)])
+    softmax = EdgeSoftmaxhip(adj)
+    softmax.build([placeholder(tuple(s.shape))], {}, {})
+    w = softmax.run([s])
+    spmm = MultiHeadSpMMhip(adj)
+    spmm.build([placeholder(key.shape), placeholder(tuple(w.shape))], {}, {})
+    out = spmm.run([nd.array(key, spmm.ctx), w]).asnumpy()
+    want = ref.attention_mh(adj.indptr, adj.indices, key, query, None)
+    np.testing.assert_allclose(out, want, rtol=1e-5, atol=1e-5)
