@@ -208,7 +208,7 @@ def main():
     ap.add_argument("--feat-len", type=int, default=64, help="feature length of the timed step")
     ap.add_argument("--graph", default="c2", help="named synthetic configuration (featgraph_amd.datasets.CONFIGS)")
     ap.add_argument("--only", choices=["all", "spmm", "sddmm", "sddmm_shuffled", "copy", "mh_sddmm", "mh_spmm", "mh_sddmm_softmax",
-                                       "mh_attention", "mh_attention_kv", "mh_attention_grad", "gather_probe", "gather_store_probe"],
+                                       "mh_attention", "mh_attention_kv", "mh_attention_grad", "gather_probe", "gather_store_probe", "gather_stream_probe"],
                     default="all",
                     help="spmm / sddmm / copy / gather_probe: run just that kernel (for profiler runs), no sweep, no "
                          "CPU leg; mh_sddmm / mh_spmm: the multi-head operators (8 heads of --feat-len floats, use "
@@ -365,6 +365,33 @@ def main():
         feat_t = device_normal((n_cols, F), 1)
         p = gather_probe(feat_t, nnz, args.steps, band=args.band_rows or None)
         print(json.dumps({"kernel": "gather_probe", "F": F, **(p or {})}))
+        return
+
+    if args.only == "gather_stream_probe":
+        # bare gathers of 64-float rows from a 4 MB band, with an index-like stream of 8 bytes per gather beside them
+        band = 16384
+        feat_t = device_normal((band, 64), 1)
+        stream_dw = 1 << 28                                  # 1 GiB of zeros
+        buf = torch.zeros(stream_dw, dtype=torch.int32, device=dev)
+        rows = []
+        for what, mode, window in (("gathers only", 0, 65536),
+                                   ("stream from HBM, read by every wave", 1, stream_dw),
+                                   ("stream from a 64 MB window, read by every wave", 1, 1 << 24),
+                                   ("stream from a 256 KB window, read by every wave", 1, 1 << 16),
+                                   ("stream from HBM, read by one wave of four", 2, stream_dw),
+                                   ("stream from a 256 KB window, read by one wave of four", 2, 1 << 16),
+                                   ("stream from HBM through the scalar cache", 3, stream_dw),
+                                   ("stream from a 256 KB window through the scalar cache", 3, 1 << 16)):
+            def go():
+                return L.fg_probe_gather_stream_f32(feat_t.data_ptr(), band, nnz, buf.data_ptr(), stream_dw, window, mode,
+                                                    sink.data_ptr(), stream.cuda_stream)
+            issued = go()
+            if issued <= 0:
+                raise RuntimeError(L.fg_last_error().decode("utf-8", "replace"))
+            ms = timed(go, args.steps, 2) * nnz / issued
+            rows.append({"variant": what, "ms_per_%d_gathers" % nnz: round(ms, 4)})
+            log("%-56s %.3f ms" % (what, ms))
+        print(json.dumps({"kernel": "gather_stream_probe", "band_rows": band, "row_floats": 64, "rows": rows}))
         return
 
     if args.only == "gather_store_probe":

@@ -47,6 +47,7 @@ SIGNATURES = {
     "fg_probe_gather_write_rows_f32": (ctypes.c_int, [_p, _i64, _i32, _i64, _i32, _p, _i64, _p, _p]),
     "fg_probe_gather_write_rows_count": (ctypes.c_int, [_i32, _i64, _i32, _p, _p]),
     "fg_probe_store_rows_f32": (_i64, [_p, _i64, _i32, _i64, _p]),
+    "fg_probe_gather_stream_f32": (_i64, [_p, _i32, _i64, _p, _i64, _i64, _i32, _p, _p]),
     "fg_config_set": (ctypes.c_int, [ctypes.c_char_p, _i32]),
     "fg_config_get": (ctypes.c_int, [ctypes.c_char_p, ctypes.POINTER(_i32)]),
     "fg_spmm_describe": (ctypes.c_int, [_p, _i32, _i32, _i32, ctypes.c_char_p, _i64]),

@@ -131,6 +131,76 @@ bool rows_shape(int32_t row_floats, int *lpr, int *nv, int64_t *per_iter) {
   return true;
 }
 
+// The gather pattern of probe_gather_kernel (64-float tiles, one 4 MB band) with an id / value-like stream beside
+// it: 8 bytes per gathered row, read from `stream` at addresses no wave shares, wrapped into a window of
+// window_dw dwords (the whole buffer: every piece comes from HBM; 64 MB: the Infinity Cache holds it; 256 KB: L2
+// does).  MODE 1: every wave reads its own piece (512 bytes per sixteen gather instructions) with one vector load,
+// requested an iteration ahead and mixed into the next iteration's row numbers, as an operator's ids are.
+// MODE 2: the first wave of every workgroup reads the pieces of all four and gathers nothing; the other three
+// gather a third more each.  MODE 3: as MODE 1 through the scalar cache (wave-uniform address).
+template <int MODE>
+__global__ __launch_bounds__(fg::kBlockThreads) void probe_gather_stream_kernel(const float *feat, uint32_t band_rows,
+                                                                                const uint32_t *__restrict__ stream,
+                                                                                uint32_t window_dw, int iters,
+                                                                                uint32_t bytes, float *sink) {
+  constexpr int U = 16;
+  const int lane = threadIdx.x & (fg::kWaveSize - 1);
+  const int gl = lane & 15, g = lane / 16;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * fg::kWavesPerBlock + (threadIdx.x >> 6));
+  uint32_t s = wave * 2654435761u + static_cast<uint32_t>(g) * 40503u + 12345u;
+  float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(feat), 0, static_cast<int>(bytes), 0x00020000);
+  const uint32_t mask = window_dw - 1;  // a power of two
+  uint32_t id_now = 0, id_next = 0;
+  if (MODE == 2) {
+    if ((threadIdx.x >> 6) == 0) {
+      uint32_t t = 0;
+      for (int it = 0; it < iters * fg::kWavesPerBlock; it += 8) {
+        uint2 v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const uint32_t at = ((blockIdx.x * static_cast<uint32_t>(fg::kWavesPerBlock * iters) + static_cast<uint32_t>(it + k)) * 128u) & mask;
+          v[k] = *reinterpret_cast<const uint2 *>(stream + at + lane * 2);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) t += v[k].x + v[k].y;
+      }
+      if (t == 0x12345u) sink[1] = 1.0f;
+      return;
+    }
+    iters = iters * 4 / 3;
+  }
+  for (int it = 0; it < iters; ++it) {
+    const uint32_t at = ((wave * static_cast<uint32_t>(iters) + static_cast<uint32_t>(it)) * 128u) & mask;
+    if (MODE == 1) {
+      const uint2 v = *reinterpret_cast<const uint2 *>(stream + at + lane * 2);
+      id_next = v.x + v.y;
+    } else if (MODE == 3) {
+      uint32_t t = 0;
+#pragma unroll
+      for (int k = 0; k < 128; ++k) t += stream[at + k];
+      id_next = t;
+    }
+    float4 x[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      s = s * 1664525u + 1013904223u;
+      const uint32_t r = ((s >> 8) + id_now) % band_rows;
+      x[u] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, static_cast<int>(r * 256u + gl * 16u), 0, 0));
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      acc.x += x[u].x;
+      acc.y += x[u].y;
+      acc.z += x[u].z;
+      acc.w += x[u].w;
+    }
+    id_now = id_next;
+  }
+  if (acc.x + acc.y + acc.z + acc.w == __builtin_inff()) sink[0] = acc.x;
+}
+
 }  // namespace
 
 // Iterations of the grid and, with writes, iterations between a group's writes, for a request.
@@ -278,4 +348,46 @@ extern "C" int64_t fg_probe_gather_count(int64_t n_rows, int32_t tile, int32_t b
   const int64_t per_iter = int64_t{kProbeBlocks} * fg::kWavesPerBlock * (fg::kWaveSize / G) * 16;
   const int64_t iters = std::max<int64_t>(1, (n_gathers / passes + per_iter / 2) / per_iter);
   return passes * iters * per_iter;
+}
+
+// n_gathers rows of 64 floats out of the first band_rows rows of feat, with 8 bytes per gather read from
+// stream_buf beside them (mode and window as described at the kernel; mode 0: no stream).  stream_buf holds
+// stream_dwords dwords of zeros, window_dwords of which are used; both are powers of two, window_dwords >= 65536.
+// Returns the number of gathers issued (the request rounded to whole iterations of the grid), or -1.
+extern "C" int64_t fg_probe_gather_stream_f32(const float *feat, int32_t band_rows, int64_t n_gathers,
+                                              const uint32_t *stream_buf, int64_t stream_dwords, int64_t window_dwords,
+                                              int32_t mode, float *sink, void *stream) {
+  auto pow2 = [](int64_t v) { return v > 0 && (v & (v - 1)) == 0; };
+  if (!feat || !sink || band_rows < 1 || band_rows > (1 << 23) || n_gathers < 0 || mode < 0 || mode > 3) {
+    fg::fail(FG_EINVAL, "bad argument to the gather-and-stream probe");
+    return -1;
+  }
+  if (mode != 0 && (!stream_buf || !pow2(stream_dwords) || !pow2(window_dwords) || window_dwords > stream_dwords ||
+                    window_dwords < 65536 || stream_dwords > (int64_t{1} << 32) || !fg::aligned_to(stream_buf, 16))) {
+    fg::fail(FG_EINVAL, "the stream buffer and its window are powers of two of dwords, the window at least 65536");
+    return -1;
+  }
+  if (!fg::aligned_to(feat, 16)) {
+    fg::fail(FG_EINVAL, "feat must be 16-byte aligned");
+    return -1;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int blocks = kProbeBlocks;
+  const int64_t per_iter = static_cast<int64_t>(blocks) * fg::kWavesPerBlock * 4 * 16;
+  int iters = static_cast<int>(std::max<int64_t>(1, (n_gathers + per_iter / 2) / per_iter));
+  if (mode == 2) iters = (iters + 5) / 6 * 6;  // whole batches of eight pieces for the reading wave, 4/3 for the others
+  const uint32_t bytes = static_cast<uint32_t>(band_rows) * 256u;
+  const uint32_t window = static_cast<uint32_t>(mode ? window_dwords : 65536);
+  const dim3 grid(blocks), block(fg::kBlockThreads);
+  switch (mode) {
+    case 0: probe_gather_stream_kernel<0><<<grid, block, 0, st>>>(feat, band_rows, stream_buf, window, iters, bytes, sink); break;
+    case 1: probe_gather_stream_kernel<1><<<grid, block, 0, st>>>(feat, band_rows, stream_buf, window, iters, bytes, sink); break;
+    case 2: probe_gather_stream_kernel<2><<<grid, block, 0, st>>>(feat, band_rows, stream_buf, window, iters, bytes, sink); break;
+    default: probe_gather_stream_kernel<3><<<grid, block, 0, st>>>(feat, band_rows, stream_buf, window, iters, bytes, sink); break;
+  }
+  if (hipGetLastError() != hipSuccess) {
+    fg::fail(FG_EHIP, "the gather-and-stream probe did not launch");
+    return -1;
+  }
+  return static_cast<int64_t>(iters) * per_iter;
 }

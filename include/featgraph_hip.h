@@ -410,6 +410,21 @@ FG_API int fg_probe_gather_write_rows_count(int32_t row_floats, int64_t n_gather
  */
 FG_API int64_t fg_probe_store_rows_f32(float *out, int64_t n_out_rows, int32_t row_floats, int64_t n_stores,
                                        void *stream);
+/*
+ * Bare gathers of 64-float rows out of the first band_rows rows of feat (the
+ * pattern of fg_probe_gather_f32 with a 64-float tile) with an index-like
+ * stream of 8 bytes per gather read beside them from stream_buf, which holds
+ * stream_dwords zero dwords of which the first window_dwords are used (powers
+ * of two; the whole buffer: every piece comes from HBM, a small window: from
+ * the Infinity Cache or L2).  mode 0: no stream; 1: every wave reads its own
+ * piece with a vector load an iteration ahead; 2: one wave of every four reads
+ * the pieces of all four and the other three gather; 3: as 1 through the
+ * scalar cache.  Returns the gathers issued, or -1 on a bad argument.  It shows
+ * what a stream of that size costs the gathers next to it, and by which path.
+ */
+FG_API int64_t fg_probe_gather_stream_f32(const float *feat, int32_t band_rows, int64_t n_gathers,
+                                          const uint32_t *stream_buf, int64_t stream_dwords, int64_t window_dwords,
+                                          int32_t mode, float *sink, void *stream);
 
 /*
  * Launch-shape overrides for tuning and tests.  The store is process-global

@@ -118,3 +118,6 @@ def test_error_codes_of_the_later_entry_points_without_a_device():
     assert L.fg_probe_gather_write_rows_count(100, 10, 25, ctypes.byref(g), ctypes.byref(w)) == -1
     assert L.fg_attention_csr_mh_f32(None, None, None, None, None, 8, 64, None) == -1
     assert L.fg_probe_store_rows_f32(None, 4, 512, 10, None) == -1 and L.fg_probe_store_rows_f32(16, 4, 100, 10, None) == -1
+    assert L.fg_probe_gather_stream_f32(None, 16384, 10, None, 0, 0, 0, None, None) == -1            # no matrix
+    assert L.fg_probe_gather_stream_f32(16, 16384, 10, 16, 1 << 20, 3 << 16, 1, 16, None) == -1      # window not a power of two
+    assert L.fg_probe_gather_stream_f32(16, 16384, 10, 16, 1 << 20, 1 << 16, 4, 16, None) == -1      # no such mode
