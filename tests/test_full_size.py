@@ -132,10 +132,12 @@ def c3_sddmm_module(c2):
     return coo, VanillaSDDMMhip(coo)
 
 
-@pytest.mark.parametrize("F", [32, 128, 256, 512])
+@pytest.mark.parametrize("F", [32, 128, 256, 512, 30, 65, 100])
 def test_c2_spmm_bit_exact_at_every_swept_feature_length(c2, c2_spmm_module, F):
     """Covers what only happens at full size: one launch per column-block pass over every feature tile with carried
-    sums, the wider passes of the narrower tiles, more long runs than the workgroup clamp, 100 MB run tables."""
+    sums, the wider passes of the narrower tiles, more long runs than the workgroup clamp, 100 MB run tables.
+    30, 65, 100: lengths beside the sweep, where the row's end cuts a lane's four floats (30), the rest of the row
+    runs as a narrower tile in launches of its own (65) and the last tile is a partial one (100)."""
     adj, module = c2, c2_spmm_module
     n = adj.shape[0]
     _say("SpMM c2 F=%d through VanillaSpMMhip: %s" % (F, module.lower_to_ir([placeholder((n, F))], {}, {})))
@@ -148,7 +150,7 @@ def test_c2_spmm_bit_exact_at_every_swept_feature_length(c2, c2_spmm_module, F):
     assert np.array_equal(out, want)
 
 
-@pytest.mark.parametrize("F", [32, 128, 256, 512])
+@pytest.mark.parametrize("F", [32, 128, 256, 512, 30, 130])
 def test_c3_sddmm_at_every_swept_feature_length(c3_sddmm_module, F):
     coo, module = c3_sddmm_module
     n = coo.shape[0]
