@@ -195,9 +195,7 @@ bool spmm_multi_applies(const SpmmArgs &a) {
 }
 
 bool spmm_multi_general_applies(const SpmmArgs &a) {
-  return spmm_multi_applies(a) && config().spmm_buffer_loads != 0 &&
-         static_cast<int64_t>(a.n_cols) * a.F * 4 < (int64_t{1} << 32) && a.n_cols <= (1 << 24) &&
-         static_cast<int64_t>(a.F) * 4 < (1 << 24);
+  return spmm_multi_applies(a);
 }
 
 // a.n_tiles tiles of spmm_multi_tile(a.F) floats starting at tile a.tile_base (grid.y); a.runs: one pass's records.

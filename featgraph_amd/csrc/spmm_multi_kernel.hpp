@@ -486,9 +486,11 @@ int launch_multi(const SpmmArgs &a, int64_t blocks, bool buf, bool u24, hipStrea
   const int il = std::max(a.interleave_tiles, 1);
   if (a.n_tiles % il != 0) return fail(FG_EINVAL, "tile interleave %d does not divide %d tiles", il, a.n_tiles);
   const dim3 grid(static_cast<unsigned>((blocks + a.long_blocks) * il), static_cast<unsigned>(a.n_tiles / il));
-  if constexpr (RED >= 0) {  // the generalised operator comes with buffer addressing and 24-bit offsets only
-    if (!(buf && u24)) return fail(FG_EUNSUPPORTED, "the generalised rows-per-wave kernel needs a feature matrix below 4 GiB");
-    spmm_multi_kernel<G, true, true, RED, MSG><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+  if constexpr (RED >= 0) {  // the generalised operator: buffer addressing with 24-bit offsets, or 64-bit addresses
+    if (buf && u24)
+      spmm_multi_kernel<G, true, true, RED, MSG><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+    else
+      spmm_multi_kernel<G, false, false, RED, MSG><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
   } else if (buf && u24) {
     spmm_multi_kernel<G, true, true, RED, MSG><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
   } else if (buf) {
@@ -504,9 +506,11 @@ int launch_multi(const SpmmArgs &a, int64_t blocks, bool buf, bool u24, hipStrea
 template <int RED, int MSG>
 int launch_multi_general_tile(const SpmmArgs &a, int64_t blocks, hipStream_t stream) {
   const int tile = a.multi_tile ? a.multi_tile : spmm_multi_tile(a.F);
-  if (tile == 16) return launch_multi<4, RED, MSG>(a, blocks, true, true, stream);
-  if (tile == 32) return launch_multi<8, RED, MSG>(a, blocks, true, true, stream);
-  return launch_multi<16, RED, MSG>(a, blocks, true, true, stream);
+  const bool buf = static_cast<int64_t>(a.n_cols) * a.F * 4 < (int64_t{1} << 32) && config().spmm_buffer_loads != 0;
+  const bool u24 = a.n_cols <= (1 << 24) && static_cast<int64_t>(a.F) * 4 < (1 << 24);
+  if (tile == 16) return launch_multi<4, RED, MSG>(a, blocks, buf, u24, stream);
+  if (tile == 32) return launch_multi<8, RED, MSG>(a, blocks, buf, u24, stream);
+  return launch_multi<16, RED, MSG>(a, blocks, buf, u24, stream);
 }
 
 template <int MSG>

@@ -46,10 +46,8 @@ class GeneralizedSpMMhip(SpMMbase):
         plan_text = super().lower_to_ir(input_placeholders, compute_args, schedule_args)
         head = "spmm_csr_general rows=%d cols=%d nnz=%d D=%d | msg=%s reduce=%s | " % (
             self._num_rows, self._num_cols, self._nnz, D, self._msg, self._reduce)
-        # the several-rows-per-wave kernel takes the call where it takes the plain one, for feature matrices within
-        # 32-bit byte offsets
-        if ("rows-per-wave" in plan_text and self._num_cols * D * 4 < 2 ** 32 and self._num_cols <= 2 ** 24
-                and _lib.config_get("spmm.general_multi") != 0 and _lib.config_get("spmm.buffer_loads") != 0):
+        # the several-rows-per-wave kernel takes the call where it takes the plain one
+        if "rows-per-wave" in plan_text and _lib.config_get("spmm.general_multi") != 0:
             return head + ("kernel=rows-per-wave with the message and the reducer in place of the multiply-add%s | %s" % (
                 ", then one division per element" if self._reduce == "mean" else "", plan_text.split(" | ")[-1]))
         found = re.search(r"(\d+) column blocks of (\d+)", plan_text)

@@ -74,7 +74,10 @@ def test_column_block_passes_fold_in_the_same_order(msg, reduce):
         # 72 floats: a whole 64-float tile and a partial one; 24: one partial 32-float tile; 70 and 30: the row's
         # end cuts a lane's four floats.  Both kernels: the several-rows-per-wave one (also one workgroup per run
         # of 1024 nonzeros and more) and the row-slot one.
-        for F, multi in ((72, -1), (72, 0), (24, -1), (70, -1), (30, -1), (66, -1), (129, -1), (90, -1)):
+        # buffer loads off: the same kernel with 64-bit addresses, as feature matrices of 4 GiB and more take it
+        for F, multi, buffer_loads in ((72, -1, -1), (72, 0, -1), (24, -1, -1), (70, -1, -1), (30, -1, -1), (66, -1, -1),
+                                       (129, -1, -1), (90, -1, -1), (72, -1, 0), (30, -1, 0)):
+            _lib.config_set("spmm.buffer_loads", buffer_loads)
             feat = datasets.spmm_operands(adj, F)
             feat[adj.indices[adj.indptr[7]]] = np.nan         # first message of row 7 (and wherever else the vertex occurs)
             feat[adj.indices[adj.indptr[9] + 3]] = np.nan     # a later message of row 9
@@ -94,6 +97,7 @@ def test_column_block_passes_fold_in_the_same_order(msg, reduce):
         _lib.config_set("spmm.blocked", -1)
         _lib.config_set("spmm.block_cols", 0)
         _lib.config_set("spmm.general_multi", -1)
+        _lib.config_set("spmm.buffer_loads", -1)
 
 
 def test_mul_sum_is_the_vanilla_kernel_and_max_min_match_numpy(adj_127x255):
