@@ -111,6 +111,22 @@ def test_c5_multihead_spmm_d64(c4):
     assert np.array_equal(out, want)
 
 
+def test_c5_multihead_generalised_spmm_max_and_mean_d16(c4):
+    """The per-head message / reduce slots at full size: max of the weighted rows and the mean, bit-exact."""
+    from featgraph_amd.module import MultiHeadGeneralizedSpMMhip
+    adj = c4
+    n = adj.shape[0]
+    w = datasets.softmax_edge_weights(adj, 8)
+    feat = datasets.spmm_operands(adj, (8, 16))
+    for msg, reduce in (("mul", "max"), ("add", "mean")):
+        _say("multi-head generalised SpMM c5 H=8 D=16 %s / %s through MultiHeadGeneralizedSpMMhip" % (msg, reduce))
+        module = MultiHeadGeneralizedSpMMhip(adj, msg, reduce)
+        module.build([placeholder((n, 8, 16)), placeholder(w.shape)], {}, {})
+        out = module.run([nd.array(feat, module.ctx), nd.array(w, module.ctx)]).asnumpy()
+        want = ref.spmm_mh_general(adj.indptr, adj.indices, w, feat, msg, reduce)
+        assert np.array_equal(out, want)
+
+
 # ---------------------------------------------------------------- every swept feature length at full size
 def _device_normal(shape, seed, dev):
     """Seeded N(0,1) float32 operand drawn on the device (seconds faster than numpy at these sizes), plus its host copy."""
