@@ -25,6 +25,8 @@ SIGNATURES = {
     "fg_spmm_csr_mh_general_f32": (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _i32, _i32, _p]),
     "fg_edge_softmax_backward_csr_f32": (ctypes.c_int, [_i64, _p, _p, _p, _p, _i32, _p]),
     "fg_permute_rows_f32": (ctypes.c_int, [_i64, _i32, _p, _p, _p, _p]),
+    "fg_spmm_csr_pitched_f32": (ctypes.c_int, [_p, _p, _i32, _p, _p, _i32, _p]),
+    "fg_pad_rows_f32": (ctypes.c_int, [_i64, _i32, _i32, _p, _p, _p]),
     "fg_add_f32": (ctypes.c_int, [_i64, _p, _p, _p, _p]),
     "fg_sddmm_coo_general_f32": (ctypes.c_int, [_i64, _p, _p, _p, _p, _p, _i32, _i32, _p]),
     "fg_spmm_csr_mh_f32": (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _i32, _p]),
@@ -53,6 +55,8 @@ SIGNATURES = {
     "fg_spmm_describe": (ctypes.c_int, [_p, _i32, _i32, _i32, ctypes.c_char_p, _i64]),
     "fg_sddmm_describe": (ctypes.c_int, [_i64, _i32, _i32, ctypes.c_char_p, _i64]),
 }
+
+FG_EUNSUPPORTED = -4   # include/featgraph_hip.h
 
 _lib = None
 

@@ -474,6 +474,7 @@ int *config_slot(const char *key) {
   if (!strcmp(key, "sddmm.regroup")) return &c.sddmm_regroup;
   if (!strcmp(key, "sddmm.xcd")) return &c.sddmm_xcd;
   if (!strcmp(key, "spmm.xcd")) return &c.spmm_xcd;
+  if (!strcmp(key, "spmm.pad_rows")) return &c.spmm_pad_rows;
   if (!strcmp(key, "attention.blocks")) return &c.attention_blocks;
   return nullptr;
 }
@@ -648,6 +649,26 @@ int fg_spmm_csr_mh_f32(const fg_spmm_plan *plan, const float *feat, const float 
     }
   }
   return FG_OK;
+}
+
+int fg_spmm_csr_pitched_f32(const fg_spmm_plan *plan, const float *feat, int32_t feat_pitch, const float *vals,
+                            float *out, int32_t F, void *stream) {
+  if (feat_pitch < F || feat_pitch % 4 != 0)
+    return fg::fail(FG_EINVAL, "feat_pitch = %d must be a multiple of 4 and at least F = %d", feat_pitch, F);
+  fg::SpmmArgs a;
+  fg::SpmmShape s;
+  if (int rc = spmm_prepare(plan, feat, vals, out, 1, F, 0, &a, &s)) return rc;
+  const fg::MultiRuns *runs = multi_table(plan, a, 0);
+  if (!runs) return fg::fail(FG_EUNSUPPORTED, "only the several-rows-per-wave kernel reads feature rows at a pitch of their own");
+  a.feat_pitch = feat_pitch;
+  return multi_run(plan, runs, a, static_cast<hipStream_t>(stream));
+}
+
+int fg_pad_rows_f32(int64_t n, int32_t F, int32_t pitch, const float *in, float *out, void *stream) {
+  if (n < 0 || F < 1 || pitch < F) return fg::fail(FG_EINVAL, "need n >= 0 and 1 <= F <= pitch");
+  if (n == 0) return FG_OK;
+  if (!in || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
+  return fg::pad_rows_launch(in, out, n, F, pitch, static_cast<hipStream_t>(stream));
 }
 
 int fg_spmm_csr_general_f32(const fg_spmm_plan *plan, const float *feat, const float *vals, float *out, int32_t F,
@@ -1094,7 +1115,7 @@ int fg_config_set(const char *key, int32_t value) {
                     slot == &fg::config().spmm_multi || slot == &fg::config().sddmm_sorted_copy ||
                     slot == &fg::config().sddmm_regroup || slot == &fg::config().spmm_relay ||
                     slot == &fg::config().spmm_general_multi || slot == &fg::config().sddmm_xcd ||
-                    slot == &fg::config().spmm_xcd;
+                    slot == &fg::config().spmm_xcd || slot == &fg::config().spmm_pad_rows;
   // flags: 0 / 1 are explicit, anything negative restores the default;
   // sizes: 0 restores the default
   *slot = flag ? (value < 0 ? -1 : (value != 0)) : std::max(value, 0);

@@ -77,6 +77,15 @@ __global__ __launch_bounds__(kBlockThreads) void add_kernel(const float *a, cons
   for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < n; t += stride) out[t] = a[t] + b[t];
 }
 
+// out[i, 0 .. F-1] = in[i, 0 .. F-1] for rows of `pitch` floats in out (the floats behind F are left as they are)
+__global__ __launch_bounds__(kBlockThreads) void pad_rows_kernel(const float *in, float *out, int64_t n, int32_t F, int32_t pitch) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x, total = n * F;
+  for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < total; t += stride) {
+    const int64_t row = t / F;
+    out[row * pitch + (t - row * F)] = in[t];
+  }
+}
+
 unsigned grid_for(int64_t threads) {
   return static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>((threads + kBlockThreads - 1) / kBlockThreads, 1 << 16)));
 }
@@ -98,6 +107,13 @@ int edge_softmax_backward_launch(const int32_t *indptr, const float *weights, co
 int permute_rows_launch(const int32_t *perm, const float *in, float *out, int64_t n, int32_t width, hipStream_t stream) {
   if (n == 0) return FG_OK;
   permute_rows_kernel<<<dim3(grid_for(n * width)), dim3(kBlockThreads), 0, stream>>>(perm, in, out, n, width);
+  FG_HIP_TRY(hipGetLastError());
+  return FG_OK;
+}
+
+int pad_rows_launch(const float *in, float *out, int64_t n, int32_t F, int32_t pitch, hipStream_t stream) {
+  if (n == 0) return FG_OK;
+  pad_rows_kernel<<<dim3(grid_for(n * F)), dim3(kBlockThreads), 0, stream>>>(in, out, n, F, pitch);
   FG_HIP_TRY(hipGetLastError());
   return FG_OK;
 }

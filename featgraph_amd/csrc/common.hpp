@@ -30,6 +30,7 @@ struct Config {
   int sddmm_fast = -1, sddmm_buffer_loads = -1, sddmm_rows = -1, sddmm_rows_blocks = 0;
   int attention_blocks = 0, sddmm_rows_wide = 0, sddmm_sorted_copy = -1, sddmm_regroup = -1, spmm_relay = -1, spmm_general_multi = -1;
   int sddmm_xcd = -1, spmm_xcd = -1;
+  int spmm_pad_rows = -1;
 };
 Config &config();
 
@@ -70,6 +71,7 @@ struct SpmmArgs {
   int32_t long_blocks = 0;  // long_blocks workgroups of the grid
   int32_t interleave_tiles = 1;  // this many tiles alternate workgroup by workgroup along grid.x; the rest along grid.y
   int32_t multi_tile = 0;        // floats per tile of the several-rows-per-wave kernel (16 / 32 / 64); 0: by feature length
+  int32_t feat_pitch = 0;        // several-rows-per-wave kernel: floats from one feature row to the next; 0: F
   // records over a re-laid copy of the ids (MultiRuns::ids_p): `indices` is that copy, and a run's values start
   // at the CSR position in the record's fourth entry
   int32_t vals_by_csr = 0;
@@ -219,6 +221,7 @@ int edge_softmax_backward_launch(const int32_t *indptr, const float *weights, co
                                  int32_t n_rows, int32_t H, hipStream_t stream);
 int permute_rows_launch(const int32_t *perm, const float *in, float *out, int64_t n, int32_t width, hipStream_t stream);
 int add_launch(const float *a, const float *b, float *out, int64_t n, hipStream_t stream);
+int pad_rows_launch(const float *in, float *out, int64_t n, int32_t F, int32_t pitch, hipStream_t stream);
 
 // Multi-head SDDMM, edge softmax and multi-head SpMM as one kernel (attention.hip).
 bool attention_fused_applies(const float *key, const float *query, const float *value, const float *out, int32_t H,

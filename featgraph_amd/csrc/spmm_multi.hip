@@ -207,8 +207,9 @@ int spmm_multi_launch(const SpmmArgs &a, hipStream_t stream) {
   const int64_t blocks = config().spmm_multi_blocks > 0 ? config().spmm_multi_blocks : 8192;
   if (a.long_runs < 0 || a.long_runs > a.n_rows || a.long_blocks < 0 || (a.long_runs > 0) != (a.long_blocks > 0))
     return fail(FG_EINVAL, "inconsistent long-run split (%d runs, %d workgroups)", a.long_runs, a.long_blocks);
-  const bool buf = static_cast<int64_t>(a.n_cols) * a.F * 4 < (int64_t{1} << 32) && config().spmm_buffer_loads != 0;
-  const bool u24 = a.n_cols <= (1 << 24) && static_cast<int64_t>(a.F) * 4 < (1 << 24);
+  const int64_t pitch = a.feat_pitch ? a.feat_pitch : a.F;
+  const bool buf = static_cast<int64_t>(a.n_cols) * pitch * 4 < (int64_t{1} << 32) && config().spmm_buffer_loads != 0;
+  const bool u24 = a.n_cols <= (1 << 24) && pitch * 4 < (1 << 24);
   const int tile = a.multi_tile ? a.multi_tile : spmm_multi_tile(a.F);
   if (a.reduce >= 0) {
     if (!spmm_multi_general_applies(a))

@@ -329,7 +329,7 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(3
   const int shared = f0_nominal - f0;  // leading floats of the lane's four that are its neighbour's
   const int64_t F = a.F;
   const uint32_t lane_bytes = static_cast<uint32_t>(f0) * 4u;
-  const FeatRows<BUF, U24> feat(a.feat, a.n_cols, F);
+  const FeatRows<BUF, U24> feat(a.feat, a.n_cols, a.feat_pitch ? a.feat_pitch : F);
   const bool carry = a.accumulate != 0;
   // the first workgroups take the long runs (the records come by descending length), one workgroup per run
   if (bx < a.long_blocks) {
@@ -506,8 +506,9 @@ int launch_multi(const SpmmArgs &a, int64_t blocks, bool buf, bool u24, hipStrea
 template <int RED, int MSG>
 int launch_multi_general_tile(const SpmmArgs &a, int64_t blocks, hipStream_t stream) {
   const int tile = a.multi_tile ? a.multi_tile : spmm_multi_tile(a.F);
-  const bool buf = static_cast<int64_t>(a.n_cols) * a.F * 4 < (int64_t{1} << 32) && config().spmm_buffer_loads != 0;
-  const bool u24 = a.n_cols <= (1 << 24) && static_cast<int64_t>(a.F) * 4 < (1 << 24);
+  const int64_t pitch = a.feat_pitch ? a.feat_pitch : a.F;
+  const bool buf = static_cast<int64_t>(a.n_cols) * pitch * 4 < (int64_t{1} << 32) && config().spmm_buffer_loads != 0;
+  const bool u24 = a.n_cols <= (1 << 24) && pitch * 4 < (1 << 24);
   if (tile == 16) return launch_multi<4, RED, MSG>(a, blocks, buf, u24, stream);
   if (tile == 32) return launch_multi<8, RED, MSG>(a, blocks, buf, u24, stream);
   return launch_multi<16, RED, MSG>(a, blocks, buf, u24, stream);

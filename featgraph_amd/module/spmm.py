@@ -132,21 +132,54 @@ class SpMMbase:
         self._H, self._D, self._feat_tiles = H, D, tiles
         out_shape = (self._num_rows,) + tuple(shapes[0][1:])
         self.out_tvm = NDArray(torch.zeros(out_shape, dtype=torch.float32, device=self._ctx))
+        self._padded = None
+        pitch = self._row_pitch(H, D, tiles)
+        if pitch:
+            self._padded = torch.zeros((self._num_cols, pitch), dtype=torch.float32, device=self._ctx)
         self._built = True
+
+    _pads_rows = False
+
+    def _describe(self, H, D, tiles):
+        buf = ctypes.create_string_buffer(1024)
+        _lib.check(_lib.lib().fg_spmm_describe(self._plan, H, D, tiles, buf, len(buf)))
+        return buf.value.decode()
+
+    def _row_pitch(self, H, D, tiles):
+        """Floats per row of the padded copy of the features that a run gathers from, or 0 for none.  A feature row
+        whose byte length is not a multiple of the 128-byte cache line makes every 256-byte piece that is gathered
+        lie across three lines instead of two; for rows beyond 64 floats a copy with rows padded to a multiple of 32
+        floats, made at every run, costs far less than that (232,965 x 100 floats: 0.05 ms against 1.2 ms; up to 64
+        floats the copy costs what it saves).  Only the
+        several-rows-per-wave kernel reads rows at a pitch."""
+        if not self._pads_rows or H != 1 or tiles or D <= 64 or D % 32 == 0 or _lib.config_get("spmm.pad_rows") == 0:
+            return 0
+        return (D + 31) // 32 * 32 if "rows-per-wave" in self._describe(H, D, tiles) else 0
 
     def lower_to_ir(self, input_placeholders, compute_args, schedule_args):
         """Description of the launch that `build` with these arguments would use (module/spmm.py:113-140
         returns TVM IR; the kernels here are prebuilt, so the plan is what there is to inspect)."""
         _, H, D, tiles = self._parse_build(input_placeholders, compute_args, schedule_args)
-        buf = ctypes.create_string_buffer(1024)
-        _lib.check(_lib.lib().fg_spmm_describe(self._plan, H, D, tiles, buf, len(buf)))
-        return buf.value.decode()
+        text = self._describe(H, D, tiles)
+        pitch = self._row_pitch(H, D, tiles)
+        return text + (" | feature rows copied to a pitch of %d floats at every run" % pitch if pitch else "")
 
     def _launch(self, tensors):
         feat = tensors[0]
+        stream = C.current_stream_handle(self._ctx)
+        if self._padded is not None:
+            pitch = self._padded.shape[1]
+            _lib.check(_lib.lib().fg_pad_rows_f32(self._num_cols, self._D, pitch, feat.data_ptr(),
+                                                  self._padded.data_ptr(), stream))
+            status = _lib.lib().fg_spmm_csr_pitched_f32(
+                self._plan, self._padded.data_ptr(), pitch, self._adj_vals_dev.data_ptr(),
+                self.out_tvm.tensor.data_ptr(), self._D, stream)
+            if status != _lib.FG_EUNSUPPORTED:        # a tuning key switched the kernel off after build: the plain call
+                _lib.check(status)
+                return
         _lib.check(_lib.lib().fg_spmm_csr_f32(
             self._plan, feat.data_ptr(), self._adj_vals_dev.data_ptr(), self.out_tvm.tensor.data_ptr(),
-            self._D, self._feat_tiles, C.current_stream_handle(self._ctx)))
+            self._D, self._feat_tiles, stream))
 
     def _checked_inputs(self, input_ndarrays):
         if not self._built:
@@ -189,6 +222,8 @@ class SpMMbase:
 class VanillaSpMMhip(SpMMbase):
     """CSR SpMM on the GPU.  VanillaSpMMhip(adj) is the call of VanillaSpMMcuda (module/spmm.py:212-214);
     the optional num_col_partitions is the argument of VanillaSpMMx86 (:198)."""
+
+    _pads_rows = True
 
     def __init__(self, adj_scipy, num_col_partitions=None):
         super().__init__(adj_scipy, num_col_partitions)

@@ -97,6 +97,23 @@ FG_API int fg_spmm_plan_row_order(const fg_spmm_plan *plan, int32_t *row_order_h
  */
 FG_API int fg_spmm_csr_f32(const fg_spmm_plan *plan, const float *feat, const float *vals, float *out, int32_t F,
                     int32_t feat_tiles, void *stream);
+/*
+ * fg_spmm_csr_f32 over a feature matrix whose rows lie feat_pitch floats apart
+ * (feat_pitch >= F, a multiple of 4; out keeps rows of F floats).  No
+ * counterpart in the reference: a 256-byte piece of a row whose byte length is
+ * not a multiple of the 128-byte cache line lies across three lines instead of
+ * two, which costs gathers up to half as much again (100 floats against 128:
+ * 4.7 against 3.4 ms on the 114.6M-nonzero graph); a caller that can afford a
+ * copy of the features with rows padded to a multiple of 32 floats
+ * (fg_pad_rows_f32) runs this entry point over the copy.  FG_EUNSUPPORTED when
+ * the several-rows-per-wave kernel, the only one that takes a pitch, does not
+ * take the call (then call fg_spmm_csr_f32 on the matrix itself).  Bit-identical
+ * to fg_spmm_csr_f32.
+ */
+FG_API int fg_spmm_csr_pitched_f32(const fg_spmm_plan *plan, const float *feat, int32_t feat_pitch, const float *vals,
+                                   float *out, int32_t F, void *stream);
+/* out[i * pitch + k] = in[i * F + k] for i < n, k < F; the floats behind F in a row of out are left as they are. */
+FG_API int fg_pad_rows_f32(int64_t n, int32_t F, int32_t pitch, const float *in, float *out, void *stream);
 
 /*
  * fg_spmm_csr_f32 without a plan and without any allocation.  No counterpart in
@@ -473,6 +490,10 @@ FG_API int64_t fg_probe_gather_stream_f32(const float *feat, int32_t band_rows, 
  * the band of its own pass -- and whether the library's own blocks come in a
  * multiple of eight passes; read at plan creation and at launch; default 1;
  * same result bits either way),
+ * "spmm.pad_rows" (0/1: whether VanillaSpMMhip, the Python module, gathers from
+ * a copy of the features with rows padded to a multiple of 32 floats when the
+ * feature length is beyond 64 floats and not one, fg_spmm_csr_pitched_f32; the C entry points do
+ * not read it; default 1),
  * "attention.blocks" (grid size of the fused attention kernel; by default one
  * vertex row per wave when a row is 1 KB or more, else 65536 workgroups that
  * walk the rows).  Value 0 restores the default of a size; for the 0/1 flags a

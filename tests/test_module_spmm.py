@@ -39,7 +39,7 @@ def config_guard():
                 "spmm.multi_blocks", "spmm.multi_long", "spmm.tile_interleave"):
         _lib.config_set(key, 0)
     for key in ("spmm.sorted", "spmm.blocked", "spmm.pipeline",
-                "spmm.buffer_loads", "spmm.multi", "spmm.relay"):
+                "spmm.buffer_loads", "spmm.multi", "spmm.relay", "spmm.pad_rows"):
         _lib.config_set(key, -1)
 
 
@@ -297,6 +297,37 @@ def test_rows_per_wave_kernel_gives_the_same_bits(config_guard, blocks, long_run
         module.out_tvm.tensor.fill_(3.0)               # stale contents must not leak into the carried sums
         out = module.run([nd.array(feat, module.ctx)]).asnumpy()
         assert np.array_equal(out, _oracle(adj, feat)), "F=%d" % F
+
+
+@pytest.mark.parametrize("blocked", [0, 1])
+def test_feature_rows_that_are_not_a_multiple_of_a_cache_line_are_gathered_from_a_padded_copy(config_guard, blocked):
+    """VanillaSpMMhip copies feature rows of more than 64 floats whose length is not a multiple of 32 to rows that
+    are, at every run, and gathers from the copy (fg_pad_rows_f32, fg_spmm_csr_pitched_f32): the same bits, for the
+    second run's features as for the first's, with the copy switched off, and when the kernel that reads a pitch is
+    switched off after build."""
+    adj = datasets.config_graph("c2-mini")
+    _lib.config_set("spmm.blocked", blocked)
+    _lib.config_set("spmm.block_cols", 700 if blocked else 0)
+    module = VanillaSpMMhip(adj)
+    for F, pitch in ((65, 96), (100, 128), (172, 192), (250, 256), (96, 0), (30, 0), (40, 0)):
+        ph = [placeholder((adj.shape[1], F))]
+        text = module.lower_to_ir(ph, {}, {})
+        assert ("pitch of %d floats" % pitch in text) if pitch else ("pitch of" not in text), text
+        module.build(ph, {}, {})
+        for seed in (1, 2):
+            feat = np.random.default_rng(seed).standard_normal((adj.shape[1], F), dtype=np.float32)
+            module.out_tvm.tensor.fill_(5.0)
+            assert np.array_equal(module.run([nd.array(feat, module.ctx)]).asnumpy(), _oracle(adj, feat)), (F, seed)
+        _lib.config_set("spmm.multi", 0)                  # after build: the pitched call is refused, the plain one runs
+        assert np.array_equal(module.run([nd.array(feat, module.ctx)]).asnumpy(), _oracle(adj, feat)), F
+        _lib.config_set("spmm.multi", -1)
+    _lib.config_set("spmm.pad_rows", 0)
+    ph = [placeholder((adj.shape[1], 100))]
+    assert "pitch of" not in module.lower_to_ir(ph, {}, {})
+    module.build(ph, {}, {})
+    feat = datasets.spmm_operands(adj, 100)
+    assert np.array_equal(module.run([nd.array(feat, module.ctx)]).asnumpy(), _oracle(adj, feat))
+    _lib.config_set("spmm.pad_rows", -1)
 
 
 def test_rows_per_wave_kernel_only_where_it_applies(config_guard, adj_127x255):
