@@ -27,6 +27,7 @@ SIGNATURES = {
     "fg_permute_rows_f32": (ctypes.c_int, [_i64, _i32, _p, _p, _p, _p]),
     "fg_spmm_csr_pitched_f32": (ctypes.c_int, [_p, _p, _i32, _p, _p, _i32, _p]),
     "fg_pad_rows_f32": (ctypes.c_int, [_i64, _i32, _i32, _p, _p, _p]),
+    "fg_sddmm_coo_plan_pitched_f32": (ctypes.c_int, [_p, _p, _p, _i32, _p, _i32, _p]),
     "fg_add_f32": (ctypes.c_int, [_i64, _p, _p, _p, _p]),
     "fg_sddmm_coo_general_f32": (ctypes.c_int, [_i64, _p, _p, _p, _p, _p, _i32, _i32, _p]),
     "fg_spmm_csr_mh_f32": (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _i32, _p]),

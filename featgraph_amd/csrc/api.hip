@@ -951,24 +951,40 @@ static bool sddmm_use_row_runs(const fg_sddmm_plan *plan, const float *src, cons
   return fg::config().sddmm_blocked > 0 || D >= 16;  // shorter rows leave most lanes of a 4-lane group idle
 }
 
+// the row-run kernel over feature rows that lie `pitch` floats apart
+static int sddmm_row_runs(const fg_sddmm_plan *plan, const float *src, const float *dst, float *out, int32_t D,
+                          int32_t pitch, void *stream) {
+  if (int rc = check_heads(1, D)) return rc;
+  if (!src || !dst || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
+  const fg_spmm_plan *r = plan->rows;
+  const bool copy = plan->sorted.col_s != nullptr;
+  if (int rc = fg::sddmm_rows_launch(r->seg, r->row_order, static_cast<int32_t>(r->n_rows), r->n_blocks,
+                                     sddmm_rows_merge64(plan), sddmm_rows_max_wide(plan),
+                                     copy ? plan->sorted.col_s : plan->col, src, dst, copy ? plan->sorted.results : out,
+                                     plan->n_cols * int64_t{pitch} * 4, plan->n_rows * int64_t{pitch} * 4, D, pitch,
+                                     static_cast<hipStream_t>(stream)))
+    return rc;
+  return copy ? fg::sddmm_unsort_launch(plan->sorted, plan->nnz, out, static_cast<hipStream_t>(stream)) : FG_OK;
+}
+
+int fg_sddmm_coo_plan_pitched_f32(const fg_sddmm_plan *plan, const float *src, const float *dst, int32_t pitch, float *out,
+                                  int32_t F, void *stream) {
+  if (!plan) return fg::fail(FG_EINVAL, "plan is null");
+  if (pitch < F || pitch % 4 != 0)
+    return fg::fail(FG_EINVAL, "pitch = %d must be a multiple of 4 and at least F = %d", pitch, F);
+  if (plan->nnz > 0)
+    if (int rc = check_device(plan->device)) return rc;
+  if (!sddmm_use_row_runs(plan, src, dst, 1, F))
+    return fg::fail(FG_EUNSUPPORTED, "only the row-run kernel reads feature rows at a pitch of their own");
+  return sddmm_row_runs(plan, src, dst, out, F, pitch, stream);
+}
+
 int fg_sddmm_coo_plan_f32(const fg_sddmm_plan *plan, const float *src, const float *dst, float *out, int32_t H,
                           int32_t D, void *stream) {
   if (!plan) return fg::fail(FG_EINVAL, "plan is null");
   if (plan->nnz > 0)
     if (int rc = check_device(plan->device)) return rc;
-  if (sddmm_use_row_runs(plan, src, dst, H, D)) {
-    if (int rc = check_heads(H, D)) return rc;
-    if (!src || !dst || !out) return fg::fail(FG_EINVAL, "a data pointer is null");
-    const fg_spmm_plan *r = plan->rows;
-    const bool copy = plan->sorted.col_s != nullptr;
-    if (int rc = fg::sddmm_rows_launch(r->seg, r->row_order, static_cast<int32_t>(r->n_rows), r->n_blocks,
-                                       sddmm_rows_merge64(plan), sddmm_rows_max_wide(plan),
-                                       copy ? plan->sorted.col_s : plan->col, src, dst,
-                                       copy ? plan->sorted.results : out, plan->n_cols * int64_t{D} * 4,
-                                       plan->n_rows * int64_t{D} * 4, D, static_cast<hipStream_t>(stream)))
-      return rc;
-    return copy ? fg::sddmm_unsort_launch(plan->sorted, plan->nnz, out, static_cast<hipStream_t>(stream)) : FG_OK;
-  }
+  if (sddmm_use_row_runs(plan, src, dst, H, D)) return sddmm_row_runs(plan, src, dst, out, D, D, stream);
   if (!sddmm_use_blocks(plan, src, dst, H, D)) {
     fg::SddmmArgs a;
     fg::SddmmShape s;

@@ -189,7 +189,7 @@ int sddmm_tile_launch(const int32_t *row_p, const int32_t *col_p, const int32_t 
 int sddmm_rows_tile(int32_t F, int max_wide);
 int sddmm_rows_launch(const int32_t *seg, const int32_t *row_order, int32_t n_rows, int32_t n_blocks, int32_t merge64,
                       int max_wide, const int32_t *col, const float *src, const float *dst, float *out,
-                      int64_t src_bytes, int64_t dst_bytes, int32_t F, hipStream_t stream);
+                      int64_t src_bytes, int64_t dst_bytes, int32_t F, int32_t pitch, hipStream_t stream);
 // The same schedule for the elementwise edge functions (op: FG_EDGE_ADD .. FG_EDGE_DIV), out [nnz, F].
 int sddmm_rows_elementwise_launch(const int32_t *seg, const int32_t *row_order, int32_t n_rows, int32_t n_blocks,
                                   int32_t merge64, const int32_t *col, const float *src, const float *dst, float *out,

@@ -247,6 +247,7 @@ struct RowsArgs {
   float *out;
   int64_t src_bytes, dst_bytes;
   int32_t n_rows, F;
+  int32_t pitch;             // floats from one row of src / dst to the next (F unless the caller padded the rows)
   int32_t first, valid;      // the tile this launch covers
   int32_t n_blocks, merge;   // column blocks in the table; a pass covers `merge` neighbouring ones
   // Passes pinned to the dies: workgroup x of a launch runs on die x % 8, so the workgroups x % 8 == d take the
@@ -289,7 +290,7 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_rows_kernel(const RowsArg
   const int32_t *const seg_lo = a.seg + static_cast<int64_t>(pass) * a.merge * n;
   const int32_t *const seg_hi = a.seg + static_cast<int64_t>(min((pass + 1) * a.merge, a.n_blocks)) * n;
   const VertexRows<BUF> src(a.src, a.src_bytes), dst(a.dst, a.dst_bytes);
-  const uint32_t row_bytes = static_cast<uint32_t>(a.F) * 4u;
+  const uint32_t row_bytes = static_cast<uint32_t>(a.pitch) * 4u;
   // piece k of this lane covers floats first + 64 k + 4 gl ..; lanes past the tile's end re-read its last
   // four floats and contribute zero
   bool kok[NT];
@@ -447,7 +448,7 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_rows_elementwise_kernel(c
   const int32_t *const seg_lo = a.seg + static_cast<int64_t>(pass) * a.merge * n;
   const int32_t *const seg_hi = a.seg + static_cast<int64_t>(min((pass + 1) * a.merge, a.n_blocks)) * n;
   const VertexRows<BUF> src(a.src, a.src_bytes), dst(a.dst, a.dst_bytes);
-  const uint32_t row_bytes = static_cast<uint32_t>(a.F) * 4u;
+  const uint32_t row_bytes = static_cast<uint32_t>(a.pitch) * 4u;
   const bool kok = gl * 4 < a.valid;  // lanes past the tile's end re-read its last four floats and store nothing
   const uint32_t lane_bytes = static_cast<uint32_t>(a.first + (kok ? gl * 4 : a.valid - 4)) * 4u;
   float *const out_lane = a.out + a.first + gl * 4;
@@ -665,7 +666,7 @@ static void rows_dispatch(const RowsArgs &a, bool acc, bool buf, dim3 grid, hipS
 int sddmm_rows_tile(int32_t F, int max_wide) {
   if (F <= 16) return 16;
   if (F <= 32) return 32;
-  if (max_wide >= 2 && F >= 128) return 128;
+  if (max_wide >= 2 && F > 96) return 128;  // 97 .. 127 floats: one partly filled wide tile beats two 64-float launches
   return 64;
 }
 
@@ -682,9 +683,10 @@ static dim3 rows_grid(RowsArgs &a, int64_t blocks, int passes) {
 
 int sddmm_rows_launch(const int32_t *seg, const int32_t *row_order, int32_t n_rows, int32_t n_blocks, int32_t merge64,
                       int max_wide, const int32_t *col, const float *src, const float *dst, float *out,
-                      int64_t src_bytes, int64_t dst_bytes, int32_t F, hipStream_t stream) {
+                      int64_t src_bytes, int64_t dst_bytes, int32_t F, int32_t pitch, hipStream_t stream) {
   if (n_rows == 0) return FG_OK;
   RowsArgs a;
+  a.pitch = pitch;
   a.seg = seg;
   a.row_order = row_order;
   a.col = col;
@@ -747,6 +749,7 @@ int sddmm_rows_elementwise_launch(const int32_t *seg, const int32_t *row_order, 
   if (n_rows == 0) return FG_OK;
   if (op < FG_EDGE_ADD || op > FG_EDGE_DIV) return fail(FG_EINVAL, "edge_op = %d is not an elementwise FG_EDGE_* code", op);
   RowsArgs a;
+  a.pitch = F;
   a.seg = seg;
   a.row_order = row_order;
   a.col = col;

@@ -122,20 +122,50 @@ class SDDMMbase:
         self._H, self._D = H, D
         out_shape = (self._nnz,) if len(shapes[0]) == 2 else (self._nnz, H)
         self.out_tvm = NDArray(torch.zeros(out_shape, dtype=torch.float32, device=self._ctx))
+        self._padded = None
+        pitch = self._row_pitch(shapes, H, D)
+        if pitch:
+            self._padded = (torch.zeros((self._num_cols, pitch), dtype=torch.float32, device=self._ctx),
+                            torch.zeros((self._num_rows, pitch), dtype=torch.float32, device=self._ctx))
         self._built = True
 
-    def lower_to_ir(self, input_placeholders, compute_args, schedule_args):
-        """Description of the launch (module/sddmm.py:94-113 returns TVM IR)."""
-        _, H, D = self._parse_build(input_placeholders, compute_args, schedule_args)
+    _pads_rows = False
+
+    def _describe(self, H, D):
         buf = ctypes.create_string_buffer(1024)
         _lib.check(_lib.lib().fg_sddmm_plan_describe(self._plan, H, D, buf, len(buf)))
         return buf.value.decode()
 
+    def _row_pitch(self, shapes, H, D):
+        """Floats per row of the padded copies of both feature matrices that a run gathers from, or 0 for none: rows
+        beyond 64 floats whose length is not a multiple of 32 floats (a 128-byte cache line) are copied at every run
+        to rows that are, as VanillaSpMMhip does.  Only the row-run kernel reads rows at a pitch."""
+        if (not self._pads_rows or len(shapes[0]) != 2 or H != 1 or D <= 64 or D % 32 == 0
+                or _lib.config_get("spmm.pad_rows") == 0):
+            return 0
+        return (D + 31) // 32 * 32 if "row runs" in self._describe(H, D) else 0
+
+    def lower_to_ir(self, input_placeholders, compute_args, schedule_args):
+        """Description of the launch (module/sddmm.py:94-113 returns TVM IR)."""
+        shapes, H, D = self._parse_build(input_placeholders, compute_args, schedule_args)
+        pitch = self._row_pitch(shapes, H, D)
+        return self._describe(H, D) + (" | feature rows copied to a pitch of %d floats at every run" % pitch if pitch else "")
+
     def _launch(self, tensors):
         src, dst = tensors
+        stream = C.current_stream_handle(self._ctx)
+        if self._padded is not None:
+            src_p, dst_p = self._padded
+            pitch = src_p.shape[1]
+            _lib.check(_lib.lib().fg_pad_rows_f32(self._num_cols, self._D, pitch, src.data_ptr(), src_p.data_ptr(), stream))
+            _lib.check(_lib.lib().fg_pad_rows_f32(self._num_rows, self._D, pitch, dst.data_ptr(), dst_p.data_ptr(), stream))
+            status = _lib.lib().fg_sddmm_coo_plan_pitched_f32(
+                self._plan, src_p.data_ptr(), dst_p.data_ptr(), pitch, self.out_tvm.tensor.data_ptr(), self._D, stream)
+            if status != _lib.FG_EUNSUPPORTED:        # a tuning key switched the kernel off after build: the plain call
+                _lib.check(status)
+                return
         _lib.check(_lib.lib().fg_sddmm_coo_plan_f32(
-            self._plan, src.data_ptr(), dst.data_ptr(), self.out_tvm.tensor.data_ptr(), self._H, self._D,
-            C.current_stream_handle(self._ctx)))
+            self._plan, src.data_ptr(), dst.data_ptr(), self.out_tvm.tensor.data_ptr(), self._H, self._D, stream))
 
     def _checked_inputs(self, input_ndarrays):
         if not self._built:
@@ -180,6 +210,8 @@ class SDDMMbase:
 class VanillaSDDMMhip(SDDMMbase):
     """COO SDDMM on the GPU.  VanillaSDDMMhip(adj) is the call of VanillaSDDMMcuda (module/sddmm.py:179-181);
     the optional partition counts are the arguments of VanillaSDDMMx86 (:169)."""
+
+    _pads_rows = True
 
     def __init__(self, adj_scipy, num_row_partitions=None, num_col_partitions=None):
         super().__init__(adj_scipy, num_row_partitions, num_col_partitions)

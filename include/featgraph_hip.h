@@ -264,6 +264,16 @@ FG_API void fg_sddmm_plan_destroy(fg_sddmm_plan *plan);
  */
 FG_API int fg_sddmm_coo_plan_f32(const fg_sddmm_plan *plan, const float *src, const float *dst, float *out, int32_t H,
                                  int32_t D, void *stream);
+/*
+ * fg_sddmm_coo_plan_f32 (single head) over src and dst matrices whose rows lie
+ * `pitch` floats apart (pitch >= F, a multiple of 4), for the same reason as
+ * fg_spmm_csr_pitched_f32: rows that are not a multiple of the 128-byte cache
+ * line cost the gathers up to a third as much again.  FG_EUNSUPPORTED when the
+ * row-run kernel, the only one that takes a pitch, does not take the call.
+ * The same result bits as fg_sddmm_coo_plan_f32.  No counterpart in the reference.
+ */
+FG_API int fg_sddmm_coo_plan_pitched_f32(const fg_sddmm_plan *plan, const float *src, const float *dst, int32_t pitch,
+                                         float *out, int32_t F, void *stream);
 FG_API int fg_sddmm_plan_describe(const fg_sddmm_plan *plan, int32_t H, int32_t D, char *buf, int64_t cap);
 
 /*
@@ -490,9 +500,10 @@ FG_API int64_t fg_probe_gather_stream_f32(const float *feat, int32_t band_rows, 
  * the band of its own pass -- and whether the library's own blocks come in a
  * multiple of eight passes; read at plan creation and at launch; default 1;
  * same result bits either way),
- * "spmm.pad_rows" (0/1: whether VanillaSpMMhip, the Python module, gathers from
+ * "spmm.pad_rows" (0/1: whether VanillaSpMMhip and VanillaSDDMMhip, the Python modules, gather from
  * a copy of the features with rows padded to a multiple of 32 floats when the
- * feature length is beyond 64 floats and not one, fg_spmm_csr_pitched_f32; the C entry points do
+ * feature length is beyond 64 floats and not one, fg_spmm_csr_pitched_f32 /
+ * fg_sddmm_coo_plan_pitched_f32; the C entry points do
  * not read it; default 1),
  * "attention.blocks" (grid size of the fused attention kernel; by default one
  * vertex row per wave when a row is 1 KB or more, else 65536 workgroups that

@@ -107,6 +107,7 @@ def test_error_codes_of_the_later_entry_points_without_a_device():
     assert L.fg_spmm_csr_pitched_f32(None, 8, 128, 8, 8, 100, None) == -1                 # no plan
     assert L.fg_pad_rows_f32(4, 100, 96, 8, 8, None) == -1                                # pitch below F
     assert L.fg_pad_rows_f32(0, 100, 128, None, None, None) == 0
+    assert L.fg_sddmm_coo_plan_pitched_f32(None, 8, 8, 128, 8, 100, None) == -1            # no plan
     # gather probes
     assert L.fg_probe_gather_f32(None, 4, 64, 64, 16384, 0, None, None) == -1
     assert L.fg_probe_gather_f32(8, 4, 60, 64, 16384, 0, 8, None) == -1                  # F not a multiple of the tile

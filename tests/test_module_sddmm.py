@@ -34,7 +34,7 @@ def config_guard():
     _lib.config_set("sddmm.rows_blocks", 0)
     _lib.config_set("sddmm.rows_wide", 0)
     for key in ("sddmm.blocked", "sddmm.fast", "sddmm.buffer_loads", "sddmm.rows", "sddmm.sorted_copy", "sddmm.regroup",
-                "sddmm.xcd"):
+                "sddmm.xcd", "spmm.pad_rows"):
         _lib.config_set(key, -1)
 
 
@@ -265,6 +265,41 @@ def test_row_runs_when_the_row_end_cuts_a_lanes_piece(config_guard, F):
         isrc, idst = np.rint(src * 2), np.rint(dst * 2)
         got = module.run([nd.array(isrc, module.ctx), nd.array(idst, module.ctx)]).asnumpy()
         assert np.array_equal(got, ref.sddmm_f64(coo.row, coo.col, isrc, idst).astype(np.float32))
+
+
+def test_feature_rows_that_are_not_a_multiple_of_a_cache_line_are_gathered_from_padded_copies(config_guard):
+    """VanillaSDDMMhip copies both feature matrices to rows of a multiple of 32 floats at every run when the length
+    is beyond 64 floats and not one (fg_sddmm_coo_plan_pitched_f32): the same bits as without the copies, also for
+    the second run's operands, for a list in any order, and when the row-run kernel is switched off after build."""
+    csr = datasets.config_graph("c2-mini").tocsr()
+    coo = csr.tocoo()
+    perm = np.random.default_rng(8).permutation(coo.nnz)
+    shuffled = scipy.sparse.coo_matrix((coo.data[perm], (coo.row[perm], coo.col[perm])), shape=coo.shape)
+    _lib.config_set("sddmm.blocked", 1)
+    _lib.config_set("sddmm.block_cols", 700)
+    for adj in (coo, shuffled):
+        for F, pitch in ((100, 128), (172, 192), (65, 96), (96, 0), (40, 0)):
+            src, dst = datasets.sddmm_operands(adj, F)
+            ph = [placeholder(src.shape), placeholder(dst.shape)]
+            _lib.config_set("spmm.pad_rows", 0)
+            plain = VanillaSDDMMhip(adj)
+            assert "pitch of" not in plain.lower_to_ir(ph, {}, {})
+            plain.build(ph, {}, {})
+            _lib.config_set("spmm.pad_rows", -1)
+            module = VanillaSDDMMhip(adj)
+            text = module.lower_to_ir(ph, {}, {})
+            assert ("pitch of %d floats" % pitch in text) if pitch else ("pitch of" not in text), text
+            module.build(ph, {}, {})
+            for scale in (1.0, -0.5):
+                a, b = nd.array(src * np.float32(scale), module.ctx), nd.array(dst, module.ctx)
+                module.out_tvm.tensor.fill_(7.0)
+                assert np.array_equal(module.run([a, b]).asnumpy(), plain.run([a, b]).asnumpy()), (F, scale)
+            np.testing.assert_allclose(module.run([a, b]).asnumpy(), ref.sddmm_f64(adj.row, adj.col, src * np.float32(-0.5), dst),
+                                       rtol=RTOL, atol=ATOL)
+            _lib.config_set("sddmm.rows", 0)              # after build: the pitched call is refused, the plain one runs
+            np.testing.assert_allclose(module.run([a, b]).asnumpy(), ref.sddmm_f64(adj.row, adj.col, src * np.float32(-0.5), dst),
+                                       rtol=RTOL, atol=ATOL)
+            _lib.config_set("sddmm.rows", -1)
 
 
 @pytest.mark.parametrize("F", [128, 132, 192, 200, 260, 512])
