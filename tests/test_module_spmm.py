@@ -561,7 +561,7 @@ def test_random_structures_bit_exact_under_random_schedules(config_guard, seed):
     _lib.config_set("spmm.multi_blocks", int(rng.choice([0, 1, 2])))
     _lib.config_set("spmm.relay", int(seed % 3 != 0))
     module = VanillaSpMMhip(adj)
-    for F in rng.choice([1, 3, 4, 8, 12, 16, 24, 32, 48, 64, 100, 128, 192, 260], 5, replace=False):
+    for F in rng.choice([1, 3, 4, 5, 8, 12, 16, 24, 30, 32, 48, 64, 65, 67, 100, 128, 129, 192, 250, 260], 7, replace=False):
         feat = rng.standard_normal((n_cols, int(F))).astype(np.float32)
         module.build([placeholder(feat.shape)], {}, {})
         module.out_tvm.tensor.fill_(-1.0)
