@@ -145,6 +145,8 @@ def headline(result, detail_path=None):
     roof = {k: r.get(k) for k in ("bound", "achieved", "peak", "unit", "frac", "frac_bounded", "traffic",
                                   "traffic_source", "algorithmic_bytes", "kernel", "dispatches_per_launch",
                                   "hbm_frac_compulsory", "frac_of_gather_ceiling")}
+    # the bare gather pattern at the operator's own L2 hit rate with an index-like stream beside it / operator time
+    roof["frac_of_gather_and_stream_ceiling"] = r.get("frac_of_gather_and_stream_at_the_operators_l2_hit_rate")
     line = {k: result.get(k) for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
                                        "higher_is_better", "scaling", "vs_baseline", "dtype", "data", "config")}
     line["roofline"] = roof
@@ -292,6 +294,28 @@ def main():
         if p:
             p.update({"l2_hit_rate_of_the_operator": hit, "hit_rate_source": src_file})
         return p
+
+    def gather_and_stream_probe_at_hit_rate(feat_t, n_gathers, op, F):
+        """The 64-float gather pattern at the operator's own L2 hit rate (band widened as above) WITH an index-like
+        stream of 8 bytes per gather read from HBM by the gathering waves beside it (fg_probe_gather_stream_f32): what
+        the memory system does for the operator's mix of traffic and nothing else."""
+        hit, src_file = committed_hit_rate(op, args.graph, F)
+        if not hit or F != 64 or feat_t.shape[1] != 64:
+            return None
+        band = int(min(feat_t.shape[0], round(16384 / hit)))
+        stream_dw = 1 << 28
+        buf = torch.zeros(stream_dw, dtype=torch.int32, device=dev)
+
+        def go():
+            return L.fg_probe_gather_stream_f32(feat_t.data_ptr(), band, n_gathers, buf.data_ptr(), stream_dw, stream_dw, 1,
+                                                sink.data_ptr(), stream.cuda_stream)
+        issued = go()
+        if issued <= 0:
+            return None
+        ms = timed(go, 5, 2) * n_gathers / issued
+        del buf
+        return {"ms": ms, "band_rows": band, "stream_bytes_per_gather": 8, "l2_hit_rate_of_the_operator": hit,
+                "hit_rate_source": src_file}
 
     def rows_probe(feat_t, n_gathers, steps=3):
         """Milliseconds that n_gathers random whole-row gathers from feat_t take (rows of 128 .. 1024 floats)."""
@@ -588,6 +612,7 @@ def main():
     traffic, traffic_source = committed_traffic("spmm", args.graph, F)
     probe = gather_probe(feat.tensor, nnz) if args.only == "all" else None
     probe_hit = gather_probe_at_hit_rate(feat.tensor, nnz, "spmm", F) if args.only == "all" else None
+    probe_mix = gather_and_stream_probe_at_hit_rate(feat.tensor, nnz, "spmm", F) if args.only == "all" else None
     launch_text = spmm.lower_to_ir([placeholder((n_cols, F))], {}, {})
     m_pass = re.search(r"(\d+) launch", launch_text)
     launch_dispatches = int(m_pass.group(1)) if m_pass else None
@@ -603,6 +628,8 @@ def main():
         "gather_ceiling": probe, "frac_of_gather_ceiling": (probe["ms"] / ms) if probe else None,
         "gather_at_the_operators_l2_hit_rate": probe_hit,
         "frac_of_gather_at_the_operators_l2_hit_rate": (probe_hit["ms"] / ms) if probe_hit else None,
+        "gather_and_stream_at_the_operators_l2_hit_rate": probe_mix,
+        "frac_of_gather_and_stream_at_the_operators_l2_hit_rate": (probe_mix["ms"] / ms) if probe_mix else None,
         "note": "`achieved` is the gather model (no cache reuse credited): most of those bytes are served by L2 / "
                 "Infinity Cache and never reach HBM, so `frac` is not bounded by 1 on this graph; "
                 "hbm_frac_compulsory, l2_fabric_frac and the two frac_of_gather_* are (the bare gather stream with "
