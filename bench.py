@@ -12,7 +12,8 @@ between two events on the launch stream.  The LAST line of stdout is one short
 JSON object (under 1.5 KB: metric, value, roofline, cpu_baseline, parity); every
 other row (feature-length sweep, multi-head operators, probes, per-setting CPU
 timings) is printed earlier, one compact JSON object per line on stderr, and
-the whole record is also written to gpurun_out/bench_detail.json.  The record carries
+the whole record is also written to bench_detail.json in the directory that FEATGRAPH_BENCH_OUT names
+(default: bench_out/ beside this file).  The record carries
 
   value        SpMM GFLOP/s (2*nnz*F flops per step)
   roofline     `achieved` / `frac`: algorithmic gather-model bytes (nnz*(8+4F) + rows*(4+4F)) over the measured
@@ -187,11 +188,12 @@ def emit(result):
     row("launch", {"text": result.get("launch")})
     detail_path = None
     try:
-        out_dir = os.path.join(ROOT, "gpurun_out")
+        out_name = os.environ.get("FEATGRAPH_BENCH_OUT", "bench_out")
+        out_dir = out_name if os.path.isabs(out_name) else os.path.join(ROOT, out_name)
         os.makedirs(out_dir, exist_ok=True)
         with open(os.path.join(out_dir, "bench_detail.json"), "w") as f:
             json.dump(result, f, indent=1)
-        detail_path = "gpurun_out/bench_detail.json"
+        detail_path = os.path.join(out_name, "bench_detail.json")
     except OSError:
         pass
     sys.stderr.flush()

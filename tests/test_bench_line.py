@@ -41,7 +41,7 @@ def _canned():
 
 
 def test_headline_is_short_and_round_trips():
-    line = bench.headline_line(_canned(), "gpurun_out/bench_detail.json")
+    line = bench.headline_line(_canned(), "bench_out/bench_detail.json")
     assert "\n" not in line and len(line) < 1500
     got = json.loads(line)
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "dtype", "config",
