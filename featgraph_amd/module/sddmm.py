@@ -143,6 +143,11 @@ class SDDMMbase:
         if (not self._pads_rows or len(shapes[0]) != 2 or H != 1 or D <= 64 or D % 32 == 0
                 or _lib.config_get("spmm.pad_rows") == 0):
             return 0
+        if D % 32 < 4 or 96 < D < 128:
+            # measured on the 114.6M-edge graph: where the row's last four floats would lie across a line in every
+            # padded row (65 / 130 floats: 5.1 / 6.7 against 3.5 / 5.1 ms) and where one partly filled 128-float tile
+            # takes the row anyway (100 floats: 3.4 against 3.2) the two copies cost more than they save
+            return 0
         return (D + 31) // 32 * 32 if "row runs" in self._describe(H, D) else 0
 
     def lower_to_ir(self, input_placeholders, compute_args, schedule_args):

@@ -149,10 +149,15 @@ class SpMMbase:
         """Floats per row of the padded copy of the features that a run gathers from, or 0 for none.  A feature row
         whose byte length is not a multiple of the 128-byte cache line makes every 256-byte piece that is gathered
         lie across three lines instead of two; for rows beyond 64 floats a copy with rows padded to a multiple of 32
-        floats, made at every run, costs far less than that (232,965 x 100 floats: 0.05 ms against 1.2 ms; up to 64
-        floats the copy costs what it saves).  Only the
+        floats, made at every run, costs far less than that (232,965 x 100 / 250 floats: 3.6 against 4.7 ms / 7.4
+        against 12.3; up to 64 floats the copy costs what it saves).  Only the
         several-rows-per-wave kernel reads rows at a pitch."""
         if not self._pads_rows or H != 1 or tiles or D <= 64 or D % 32 == 0 or _lib.config_get("spmm.pad_rows") == 0:
+            return 0
+        if D < 128 and D % 32 < 4:
+            # the row's last four floats, which the lane that the row's end cuts reads, would lie across a line in
+            # every padded row; with a single whole tile before them that costs more than the copy saves (65 floats:
+            # 4.4 against 3.9 ms on the 114.6M-nonzero graph; 130 floats: 6.3 against 7.5)
             return 0
         return (D + 31) // 32 * 32 if "rows-per-wave" in self._describe(H, D, tiles) else 0
 

@@ -278,7 +278,7 @@ def test_feature_rows_that_are_not_a_multiple_of_a_cache_line_are_gathered_from_
     _lib.config_set("sddmm.blocked", 1)
     _lib.config_set("sddmm.block_cols", 700)
     for adj in (coo, shuffled):
-        for F, pitch in ((100, 128), (172, 192), (65, 96), (96, 0), (40, 0)):
+        for F, pitch in ((90, 96), (172, 192), (136, 160), (96, 0), (40, 0), (65, 0), (100, 0), (130, 0)):
             src, dst = datasets.sddmm_operands(adj, F)
             ph = [placeholder(src.shape), placeholder(dst.shape)]
             _lib.config_set("spmm.pad_rows", 0)

@@ -309,7 +309,7 @@ def test_feature_rows_that_are_not_a_multiple_of_a_cache_line_are_gathered_from_
     _lib.config_set("spmm.blocked", blocked)
     _lib.config_set("spmm.block_cols", 700 if blocked else 0)
     module = VanillaSpMMhip(adj)
-    for F, pitch in ((65, 96), (100, 128), (172, 192), (250, 256), (96, 0), (30, 0), (40, 0)):
+    for F, pitch in ((72, 96), (100, 128), (130, 160), (250, 256), (96, 0), (30, 0), (40, 0), (65, 0)):
         ph = [placeholder((adj.shape[1], F))]
         text = module.lower_to_ir(ph, {}, {})
         assert ("pitch of %d floats" % pitch in text) if pitch else ("pitch of" not in text), text
