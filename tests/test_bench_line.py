@@ -15,7 +15,9 @@ def _canned():
         "hbm_frac_compulsory": 0.0721234, "l2_fabric_frac": 0.655123456,
         "gather_ceiling": {"ms": 1.0, "tile": 64, "band_rows": 16384, "note": long_text},
         "frac_of_gather_ceiling": 0.5571234, "gather_at_the_operators_l2_hit_rate": {"ms": 1.3, "note": long_text},
-        "frac_of_gather_at_the_operators_l2_hit_rate": 0.72123456, "note": long_text * 3}
+        "frac_of_gather_at_the_operators_l2_hit_rate": 0.72123456,
+        "gather_and_stream_at_the_operators_l2_hit_rate": {"ms": 1.5, "note": long_text},
+        "frac_of_gather_and_stream_at_the_operators_l2_hit_rate": 0.85123456, "note": long_text * 3}
     return {
         "metric": "SpMM GFLOP/s (vanilla CSR, fp32, feat-len 64)", "value": 8171.123456, "unit": "GFLOP/s",
         "n_gpus": 1, "steps": 20, "warmup": 3, "ms_per_step": 1.7951234, "higher_is_better": True,
@@ -74,3 +76,18 @@ def test_headline_refuses_to_grow():
         assert "limit" in str(e)
     else:
         raise AssertionError("an oversized line was printed")
+
+
+def test_the_committed_counter_summaries_are_still_what_the_benchmark_reads():
+    """roofline.traffic, frac_bounded and the probes' bands come from profiles/*_counters.txt: every swept feature
+    length and multi-head row must parse, with bytes and hit rates in a plausible range."""
+    for op in ("spmm", "sddmm"):
+        for F in (32, 64, 128, 256, 512):
+            traffic, src = bench.committed_traffic(op, "c2", F)
+            hit, src2 = bench.committed_hit_rate(op, "c2", F)
+            assert src == src2 == "profiles/%s_c2_counters.txt" % op
+            assert 1e9 < traffic < 2e11 and 0.3 < hit < 1.0, (op, F, traffic, hit)
+    for kind, D in (("mh_sddmm", 16), ("mh_sddmm", 64), ("mh_spmm", 64)):
+        traffic, src = bench.committed_traffic_mh(kind, D)
+        assert src == "profiles/multihead_c4_counters.txt" and 1e10 < traffic < 5e11, (kind, D, traffic)
+    assert bench.committed_traffic("spmm", "c2", 48) == (None, None)
