@@ -254,13 +254,15 @@ FG_API int fg_sddmm_plan_create_partitioned(int64_t nnz, int64_t n_rows, int64_t
 FG_API void fg_sddmm_plan_destroy(fg_sddmm_plan *plan);
 
 /*
- * fg_sddmm_coo_mh_f32 on the plan's edge list.  With H = 1, F a multiple of 4
- * and 16-byte aligned operands a blocked plan runs one launch per 64-float
- * feature tile (each tile adds its partial dot product to Out, the reference's
- * feature tiling: op/vanilla_sddmm.py:49-60): over (row, column block) runs of
- * a row-sorted list, one Dst tile held in registers per run, or over the
- * re-ordered list; otherwise this is the plain kernel.  All agree within
- * float32 rounding.
+ * fg_sddmm_coo_mh_f32 on the plan's edge list.  With H = 1 and F >= 4 a blocked
+ * plan runs one launch per feature tile of up to 128 floats (each tile adds its
+ * partial dot product to Out, the reference's feature tiling:
+ * op/vanilla_sddmm.py:49-60) over (row, column block) runs of a row-sorted
+ * list -- the caller's own, or the plan's sorted copy of a list in any other
+ * order -- with one Dst tile held in registers per run; with F a multiple of 4
+ * and 16-byte aligned operands a plan built with sddmm.sorted_copy = 0 walks
+ * its re-ordered list instead; otherwise this is the plain kernel.  All agree
+ * within float32 rounding.
  */
 FG_API int fg_sddmm_coo_plan_f32(const fg_sddmm_plan *plan, const float *src, const float *dst, float *out, int32_t H,
                                  int32_t D, void *stream);
