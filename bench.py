@@ -724,6 +724,10 @@ def main():
                    "frac_of_gather_ceiling": p["ms"] / (sec * 1e3) if p else None,
                    "gather_at_the_operators_l2_hit_rate": ph_sddmm,
                    "frac_of_gather_at_the_operators_l2_hit_rate": ph_sddmm["ms"] / (sec * 1e3) if ph_sddmm else None}
+            pm = gather_and_stream_probe_at_hit_rate(ins[0].tensor, nnz, "sddmm", f)   # 64 floats only
+            if pm:
+                row["gather_and_stream_at_the_operators_l2_hit_rate"] = pm
+                row["frac_of_gather_and_stream_at_the_operators_l2_hit_rate"] = pm["ms"] / (sec * 1e3)
             if check:
                 out = sddmm.out_tvm.asnumpy()
                 s_h, d_h = ins[0].tensor.cpu().numpy(), ins[1].tensor.cpu().numpy()
