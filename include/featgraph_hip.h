@@ -112,7 +112,8 @@ FG_API int fg_spmm_csr_f32(const fg_spmm_plan *plan, const float *feat, const fl
  */
 FG_API int fg_spmm_csr_pitched_f32(const fg_spmm_plan *plan, const float *feat, int32_t feat_pitch, const float *vals,
                                    float *out, int32_t F, void *stream);
-/* out[i * pitch + k] = in[i * F + k] for i < n, k < F; the floats behind F in a row of out are left as they are. */
+/* out[i * pitch + k] = in[i * F + k] for i < n, k < F; the floats behind F in a row of out are left as they are
+ * (the pitched entry points never use them).  in and out must not overlap. */
 FG_API int fg_pad_rows_f32(int64_t n, int32_t F, int32_t pitch, const float *in, float *out, void *stream);
 
 /*
